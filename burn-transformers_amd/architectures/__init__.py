@@ -1,3 +1,3 @@
-"""Importing this package registers the architectures the library ships (GPT-2, Salopel, Kodatar)."""
+"""Importing this package registers the architectures the library ships (GPT-2, Salopel, Kodatar, Rotutar)."""
 
-from . import gpt2, kodatar, salopel  # noqa: F401
+from . import gpt2, kodatar, rotutar, salopel  # noqa: F401

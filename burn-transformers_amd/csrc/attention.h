@@ -33,7 +33,20 @@ struct AttnArgs {
   // a query at position p sees the keys from p - p % chunk through p (and, with a window as well,
   // only those the window also holds).
   int chunk;
+  // null, or one logit per query head that stands in every softmax's denominator beside the keys a
+  // query sees: exp(sink[head]) is added once, unscaled, with no key and no value of its own (the
+  // weights of a query's keys then add up to less than one).
+  const float* sink;
 };
+
+// What a sink adds to a softmax's denominator that is kept relative to the maximum `top`.  The plain and
+// the float32 decode kernels keep maxima as natural logarithms, the MFMA kernels in powers of two.
+__device__ __forceinline__ float bt_sink_term(const float* sink, int head, float top) {
+  return sink ? expf(sink[head] - top) : 0.f;
+}
+__device__ __forceinline__ float bt_sink_term_pow2(const float* sink, int head, float top) {
+  return sink ? exp2f(sink[head] * 1.4426950408889634f - top) : 0.f;
+}
 
 // The first position a query at `pos` sees: the later of its window's and its chunk's first key.
 // It never decreases as `pos` grows, so the first query of a run of queries has the lowest.

@@ -323,6 +323,7 @@ attention_prefill_kernel(AttnArgs a) {
     float total = l[nq];
     total += __shfl_xor(total, 16, 64);
     total += __shfl_xor(total, 32, 64);
+    total += bt_sink_term_pow2(a.sink, head, m[nq]);
     float inv = total > 0.f ? 1.0f / total : 0.f;
     if (qpos[nq] < 0) continue;
 #pragma unroll
@@ -693,7 +694,8 @@ attention_prefill_split_kernel(AttnArgs a) {
     const float mine = m[nq] == -INFINITY ? 0.f : exp2f(m[nq] - top);
     const float theirs = m_other == -INFINITY ? 0.f : exp2f(m_other - top);
     const float total = rows[nq][0] * mine + l_other * theirs;   // (whole sums: see attend_block)
-    float inv = total > 0.f ? 1.0f / total : 0.f;
+    // (with runs the sink joins the denominator once, where the runs are joined)
+    float inv = total > 0.f ? 1.0f / (total + bt_sink_term_pow2(a.sink, head, top)) : 0.f;
     if (qpos[nq] < 0) continue;
     if (runs > 1) {      // this run's share of the query's row, relative to its own maximum
       typedef __attribute__((__vector_size__(2 * sizeof(float)))) float float2v;
@@ -838,6 +840,7 @@ attention_decode_kernel(AttnArgs a) {
       }
     }
     if (splits == 1) {
+      den += top != -INFINITY ? bt_sink_term_pow2(a.sink, kv_head * group + j, top) : 0.f;
       out[activation_offset<bf16_t>(a.out_rows, a.ldo, tok, (kv_head * group + j) * HD + channel)] =
           (bf16_t)(den > 0.f ? num / den : 0.f);
     } else {     // this run's share, for attention_join_kernel
@@ -898,6 +901,7 @@ attention_join_kernel(AttnArgs a, int n_rows) {
     }
     top = new_top;
   }
+  if (top != -INFINITY) den += bt_sink_term_pow2(a.sink, head, top);
   bf16_t* out = static_cast<bf16_t*>(a.out);
 #pragma unroll
   for (int c = 0; c < NCH; ++c) {

@@ -204,6 +204,7 @@ attention_f32_mfma_kernel(AttnArgs a) {
   float total = run_sum;
   total += __shfl_xor(total, 16, 64);
   total += __shfl_xor(total, 32, 64);
+  total += bt_sink_term_pow2(a.sink, head, run_max);        // (the maximum is the same in a query's four lanes)
   if (exists) {
     float* out = static_cast<float*>(a.out) + (int64_t)(off + q0 + mine) * a.ldo + head * HD;
 #pragma unroll
@@ -330,6 +331,7 @@ attention_f32_decode_kernel(AttnArgs a) {
         den = fmaf(part_sum[w], f, den);
       }
       if (splits == 1) {
+        den += bt_sink_term(a.sink, head, top);
         out[channel] = den > 0.f ? num / den : 0.f;
       } else {                                                      // this run's share, for attention_f32_join_kernel
         mine[channel] = num;
@@ -359,6 +361,7 @@ attention_f32_join_kernel(AttnArgs a) {
       num = fmaf(runs[s * (hd + 2) + channel], f, num);
       den = fmaf(runs[s * (hd + 2) + hd + 1], f, den);
     }
+    den += bt_sink_term(a.sink, head, top);
     out[channel] = den > 0.f ? num / den : 0.f;
   }
 }

@@ -32,6 +32,8 @@ struct EmbedCall {
   float* out;
   float scale;             // multiplies the token's row (not the position's)
   float* copy;             // or null: a second place for the same rows
+  void* cast;              // or null: the same rows in the table's type, [tokens][cast_cols], zeros behind the width
+  int cast_cols;
 };
 
 struct AddNormCall {

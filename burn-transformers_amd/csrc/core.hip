@@ -26,7 +26,8 @@
 template <typename T>
 __global__ void embed_kernel(const int* __restrict__ ids, const int* __restrict__ pos,
                              const T* __restrict__ table, const T* __restrict__ positions,
-                             float* __restrict__ out, float* __restrict__ copy, float scale, int width) {
+                             float* __restrict__ out, float* __restrict__ copy, float scale, int width,
+                             T* __restrict__ cast, int cast_cols) {
   int t = blockIdx.x;
   const T* row = table + (int64_t)ids[t] * width;
   const T* prow = positions ? positions + (int64_t)pos[t] * width : nullptr;
@@ -35,20 +36,27 @@ __global__ void embed_kernel(const int* __restrict__ ids, const int* __restrict_
     if (prow) v += to_float(prow[c]);
     out[(int64_t)t * width + c] = v;
     if (copy) copy[(int64_t)t * width + c] = v;
+    if (cast) cast[(int64_t)t * cast_cols + c] = from_float<T>(v);
   }
+  if (cast)
+    for (int c = width + threadIdx.x; c < cast_cols; c += blockDim.x) cast[(int64_t)t * cast_cols + c] = from_float<T>(0.f);
 }
 
 BT_EXPORT int bt_embed(void* stream, int dtype, const int* ids, const int* pos, const void* table,
-                       const void* positions, float* out, int tokens, int width, float scale, float* copy) {
+                       const void* positions, float* out, int tokens, int width, float scale, float* copy,
+                       void* cast, int cast_cols) {
   if (tokens <= 0) return BT_OK;
   if (width <= 0) BT_REFUSE("embed: width %d must be positive", width);
+  if (cast && cast_cols < width) BT_REFUSE("embed: a copy of %d columns does not hold width %d", cast_cols, width);
   dim3 grid(tokens), block(256);
   if (dtype == 0)
     hipLaunchKernelGGL(embed_kernel<float>, grid, block, 0, (hipStream_t)stream, ids, pos,
-                       (const float*)table, (const float*)positions, out, copy, scale, width);
+                       (const float*)table, (const float*)positions, out, copy, scale, width,
+                       (float*)cast, cast_cols);
   else
     hipLaunchKernelGGL(embed_kernel<bf16_t>, grid, block, 0, (hipStream_t)stream, ids, pos,
-                       (const bf16_t*)table, (const bf16_t*)positions, out, copy, scale, width);
+                       (const bf16_t*)table, (const bf16_t*)positions, out, copy, scale, width,
+                       (bf16_t*)cast, cast_cols);
   return bt_check_launch("embed");
 }
 
@@ -514,6 +522,7 @@ attention_plain_kernel(AttnArgs a) {
     }
     __syncthreads();
   }
+  run_sum += bt_sink_term(a.sink, head, run_max);
   if ((int)threadIdx.x < hd) {
     T* o = static_cast<T*>(a.out) + (int64_t)t * a.ldo + head * hd;
     o[threadIdx.x] = from_float<T>(run_sum > 0.f ? acc / run_sum : 0.f);
@@ -1244,7 +1253,8 @@ BT_EXPORT int bt_count_tokens(void* stream, int* counts, int64_t ld, const int* 
 // The same entry points with their arguments as one structure (calls.h), for launch lists.
 // ---------------------------------------------------------------------------------------------
 BT_EXPORT int bt_embed_call(void* stream, const EmbedCall* c) {
-  return bt_embed(stream, c->dtype, c->ids, c->pos, c->table, c->positions, c->out, c->tokens, c->width, c->scale, c->copy);
+  return bt_embed(stream, c->dtype, c->ids, c->pos, c->table, c->positions, c->out, c->tokens, c->width, c->scale, c->copy,
+                  c->cast, c->cast_cols);
 }
 BT_EXPORT int bt_add_norm_call(void* stream, const AddNormCall* c) {
   return bt_add_norm(stream, c->out_dtype, c->x, c->delta, c->n_delta, c->delta_stride, c->bias, c->gamma, c->beta, c->eps,

@@ -9,6 +9,11 @@
 //     always-on expert with its sigmoid gate as weight), so that ONE product with the experts' down
 //     matrices laid side by side gives the weighted sum of their outputs; experts whose output is
 //     their input ("identity experts", the last router outputs) leave weight * h as 32-bit rows.
+// A router may differ in three ways (`score`, `group_rank`, `normalize`): scores that are the
+// logits' sigmoids instead of their softmax, a group's score that is the sum of its `group_rank` best
+// instead of its best, and weights that are the chosen experts' scores as they are instead of over
+// their sum.  The experts' activation (`act`) is silu(g) * u, or with a `limit`:
+// g' = min(g, limit), u' = clamp(u, -limit, limit), g' * sigmoid(alpha * g') * (u' + 1).
 // Ties between equal scores go to the lower index.
 #include "host.h"
 
@@ -28,6 +33,9 @@ struct RouteCall {
   const float* gate_w;      // [width] float32 or null
   float* weights;           // [tokens][experts]
   float* gate;              // [tokens]: sigmoid(gate_w . h), or null
+  int score;                // 0: softmax over all experts; 1: each logit's sigmoid
+  int group_rank;           // a group's score is the sum of its so many best (corrected) scores; 0 or 1: its best
+  int normalize;            // 1: the chosen experts' scores over their sum; 0: the scores as they are
 };
 
 // The best (value, index) of a wave; among equal values the lowest index.  Every lane gets it.
@@ -116,7 +124,7 @@ __global__ void __launch_bounds__(ROUTE_THREADS) route_kernel(RouteCall c) {
   total = wave_sum(total);
   float* weights = c.weights + (int64_t)t * c.experts;
   for (int e = lane, j = 0; e < c.experts; e += 64, ++j) {     // a lane keeps to its own experts: no other lane reads them yet
-    const float s = expf(score[e] - top_logit) / total;
+    const float s = c.score == 1 ? 1.0f / (1.0f + expf(-score[e])) : expf(score[e] - top_logit) / total;
     score[e] = s;
     choice[e] = s + (c.correction ? (j < 4 ? early_correction[j < 4 ? j : 0] : c.correction[e]) : 0.f);
   }
@@ -129,8 +137,29 @@ __global__ void __launch_bounds__(ROUTE_THREADS) route_kernel(RouteCall c) {
     // holds group g (at most 64 groups).
     const int per = c.experts / c.groups;
     float group_score = -INFINITY;
-    if (lane < c.groups)
-      for (int i = 0; i < per; ++i) group_score = fmaxf(group_score, choice[lane * per + i]);
+    if (lane < c.groups) {
+      if (c.group_rank <= 1) {
+        for (int i = 0; i < per; ++i) group_score = fmaxf(group_score, choice[lane * per + i]);
+      } else {
+        // the sum of the group's `group_rank` best: best after best, each below the one before it or
+        // an equal one at a higher index
+        float last = INFINITY;
+        int last_index = -1;
+        group_score = 0.f;
+        for (int r = 0; r < c.group_rank && r < per; ++r) {
+          float best = -INFINITY;
+          int best_index = -1;
+          for (int i = 0; i < per; ++i) {
+            const float v = choice[lane * per + i];
+            const bool left = v < last || (v == last && i > last_index);
+            if (left && (best_index < 0 || v > best)) { best = v; best_index = i; }
+          }
+          group_score += best;
+          last = best;
+          last_index = best_index;
+        }
+      }
+    }
     bool open = false;
     for (int kept = 0; kept < c.keep; ++kept) {
       float value = (lane < c.groups && !open) ? group_score : -INFINITY;
@@ -164,7 +193,7 @@ __global__ void __launch_bounds__(ROUTE_THREADS) route_kernel(RouteCall c) {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
   }
   // the one store of a lane's experts: the chosen ones' scores over their sum, zero elsewhere
-  const float inverse = 1.0f / (sum + 1e-20f);
+  const float inverse = c.normalize ? 1.0f / (sum + 1e-20f) : 1.0f;
   for (int e = lane; e < c.experts; e += 64) weights[e] = choice[e] == INFINITY ? score[e] * inverse : 0.f;
   if (c.gate_w && lane == 0) c.gate[t] = 1.0f / (1.0f + expf(-gate_sum));
 }
@@ -180,6 +209,8 @@ BT_EXPORT int bt_route_call(void* stream, const RouteCall* c) {
       BT_REFUSE("route: %d open groups of %d experts cannot give %d experts", c->keep, c->experts / c->groups, c->top);
   }
   if (c->width <= 0) BT_REFUSE("route: width %d must be positive", c->width);
+  if ((c->score != 0 && c->score != 1) || c->group_rank < 0 || (c->normalize != 0 && c->normalize != 1))
+    BT_REFUSE("route: score %d, group_rank %d, normalize %d: not a router this kernel knows", c->score, c->group_rank, c->normalize);
   if (!c->h || !c->W || !c->weights || (c->gate_w && !c->gate)) BT_REFUSE("route: missing operand");
   // (measured at 2,048 tokens of width 2,048: 32 us with sixteen waves a token, 18 with four)
   dim3 grid(c->tokens), block(c->tokens <= 256 ? ROUTE_THREADS : 256);
@@ -208,7 +239,19 @@ struct GatedExpertsCall {
   const void* h;            // [tokens][ldh]: the experts' input (read for identity experts only)
   int64_t ldh;
   float* identity_out;      // [tokens][width] float32: (sum of the identity experts' weights) * h; or null
+  int act;                  // 0: silu(g) * u; 1: min(g, limit) * sigmoid(alpha * min(g, limit)) * (clamp(u, -limit, limit) + 1)
+  float limit;
+  float alpha;
 };
+
+__device__ __forceinline__ float gated_unit(const GatedExpertsCall& c, float g, float u) {
+  if (c.act == 1) {
+    g = fminf(g, c.limit);
+    u = fminf(fmaxf(u, -c.limit), c.limit);
+    return g / (1.0f + expf(-c.alpha * g)) * (u + 1.0f);
+  }
+  return g / (1.0f + expf(-g)) * u;
+}
 
 template <typename T>
 __global__ void __launch_bounds__(256) gated_experts_kernel(GatedExpertsCall c) {
@@ -225,12 +268,12 @@ __global__ void __launch_bounds__(256) gated_experts_kernel(GatedExpertsCall c) 
       const float w = weights[e];
       if (w != 0.f) {
         const float g = to_float(gu[(int64_t)e * 2 * c.ff + i]), u = to_float(gu[(int64_t)e * 2 * c.ff + c.ff + i]);
-        out = w * (g / (1.0f + expf(-g))) * u;
+        out = w * gated_unit(c, g, u);
       }
     } else if (col < routed + c.shared_ff) {
       const int i = col - routed;
       const float g = to_float(gu[(int64_t)2 * routed + i]), u = to_float(gu[(int64_t)2 * routed + c.shared_ff + i]);
-      out = (c.gate ? c.gate[t] : 1.0f) * (g / (1.0f + expf(-g))) * u;
+      out = (c.gate ? c.gate[t] : 1.0f) * gated_unit(c, g, u);
     }
     hidden[col] = from_float<T>(out);
   }
@@ -250,7 +293,8 @@ BT_EXPORT int bt_gated_experts_call(void* stream, const GatedExpertsCall* c) {
   const int64_t columns = (int64_t)c->experts * c->ff + c->shared_ff;
   if (c->hidden_cols < columns || c->ld_hidden < c->hidden_cols || c->ld_gu < 2 * columns)
     BT_REFUSE("gated_experts: the rows do not hold the experts");
-  if (!c->gu || !c->weights || !c->hidden || (c->identity_out && (!c->h || c->width <= 0)))
+  if (c->act != 0 && c->act != 1) BT_REFUSE("gated_experts: unknown activation %d", c->act);
+  if (!c->gu || (!c->weights && c->experts + c->identity > 0) || !c->hidden || (c->identity_out && (!c->h || c->width <= 0)))
     BT_REFUSE("gated_experts: missing operand");
   // about 1,024 columns a work-group, fewer work-groups a token where there are many tokens
   int per_token = (c->hidden_cols + 1023) / 1024;

@@ -1,0 +1,262 @@
+// Kernels of mixers that are linear attention with a matrix state per head (no softmax, no cache of
+// keys): per head a state S [dim][vdim] in 32-bit that every token first lets decay per key channel
+// and then writes a rank-one update into, token after token.
+//   * keyed scan: per token and head, with a decay g [dim], a key k [dim], a value v [vdim], a query q [dim]:
+//         S <- diag(g) S;   u = v                              (plain write)
+//                           u = beta (v - S^T k)               (delta rule: what S already answers for k is taken off)
+//         S <- S + k u^T;   o = S^T q                          (the read-out sees the token's own write)
+//     How g, k and q come about is the kernel's `form`:
+//       form 0 (gated delta rule): q and k are rows of their own (heads may share them), optionally made unit
+//           vectors per head here, x / sqrt(sum x^2 + unit_eps), q times q_scale; g = exp(-exp(A_log[head]) * dt)
+//           from step sizes dt per head and key channel; beta = sigmoid(beta logit of the head)
+//       form 1 (forget gate that also decides what is written): f = lower + (1 - lower) * sigmoid(f_raw + f_bias)
+//           per head and key channel; g = f, k = 1 - f, q = silu(q_raw); no beta
+//   * head norm with a gate: every head's read-out over its root mean square over vdim, times a scale of
+//     vdim entries that the heads share, times the sigmoid of a gate's logits where there are any
+// A sequence's state lives in its slot's row of the cache's per-sequence state area; a step may bring any
+// number of a sequence's tokens, which are walked in order from the state the last step left.
+#include "host.h"
+#include "scan.h"
+
+struct KeyedScanCall {
+  int tokens, n_seqs;
+  int heads;              // heads of v, g, beta and of the state
+  int kv_heads;           // heads of q and k (form 0); head h uses h / (heads / kv_heads)
+  int dim, vdim;
+  int form;               // 0: delta rule; 1: forget gate with complement keys
+  int unit;               // form 0: 1 if q and k are made unit vectors per head here
+  float unit_eps;
+  float q_scale;          // form 0: factor on q (after the unit norm)
+  const float* q;         // [tokens][ld_q]: form 0: head j at columns j * dim; form 1: raw, head h at h * dim
+  int64_t ld_q;
+  const float* k;         // [tokens][ld_k] (form 0)
+  int64_t ld_k;
+  const float* v;         // [tokens][ld_v]: head h at columns h * vdim
+  int64_t ld_v;
+  const float* g;         // [tokens][ld_g]: head h at columns h * dim: step sizes (form 0), gate logits (form 1)
+  int64_t ld_g;
+  const float* beta;      // [tokens][ld_beta]: one logit a head (form 0)
+  int64_t ld_beta;
+  const float* A_log;     // [heads] (form 0)
+  const float* g_bias;    // [heads * dim] (form 1), or null
+  const float* lower;     // [heads * dim] (form 1)
+  float* out;             // [tokens][ld_out] float32: head h at columns h * vdim
+  int64_t ld_out;
+  float* S;               // slot s: [heads][vdim / 4 rounded up][dim][4] at S + s * state_stride
+  int64_t state_stride;
+  const int* seq_off;     // [n_seqs + 1]
+  const int* slots;       // [n_seqs]
+};
+
+// One wave per (4 value channels of a head, sequence): sixteen lanes share a channel, lane j of them owns
+// the key channels j, j + 16, ... of its column of S in registers.  A work-group is four waves with four
+// channels each of the same head: they share the run of (g, k, q) in LDS.
+#define KS_WAVES 4
+
+template <int R, int FORM>
+__global__ void __launch_bounds__(64 * KS_WAVES) keyed_scan_kernel(KeyedScanCall c, int chunk, int tiles) {
+  extern __shared__ __attribute__((aligned(16))) float lds[];
+  constexpr int NP = 16 * R;
+  float4* gkq = reinterpret_cast<float4*>(lds);                               // [chunk][NP]: decay, key, query
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, sub = lane & 15, pl = lane >> 4;
+  float2* tok = reinterpret_cast<float2*>(lds + (size_t)chunk * NP * 4) + (size_t)wave * chunk * 4;   // [waves][chunk][4]: v, beta
+  const int tile = min((int)blockIdx.x * KS_WAVES + wave, tiles - 1), head = blockIdx.y, seq = blockIdx.z;
+  const bool works = (int)blockIdx.x * KS_WAVES + wave < tiles;
+  const int p = tile * 4 + pl;
+  const bool live = works && p < c.vdim;
+  const int shared = FORM == 0 ? head / (c.heads / c.kv_heads) : head;
+  const int first = c.seq_off[seq], last = c.seq_off[seq + 1];
+  float* held = c.S + (int64_t)c.slots[seq] * c.state_stride + ((int64_t)head * tiles + tile) * c.dim * 4 + pl;
+  float S[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const int n = sub + 16 * r;
+    S[r] = n < c.dim ? held[(int64_t)n * 4] : 0.f;
+  }
+  const float rate = FORM == 0 ? -expf(c.A_log[head]) : 0.f;
+  float* ocol = c.out + head * c.vdim + (live ? p : 0);
+  for (int t0 = first; t0 < last; t0 += chunk) {
+    const int count = min(chunk, last - t0);
+    __syncthreads();
+    for (int e = threadIdx.x; e < count * NP; e += 64 * KS_WAVES) {
+      const int i = e / NP, n = e % NP;
+      float4 in = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (n < c.dim) {
+        const int64_t t = t0 + i;
+        if (FORM == 0) {
+          in.x = expf(rate * c.g[t * c.ld_g + head * c.dim + n]);
+          in.y = c.k[t * c.ld_k + shared * c.dim + n];
+          in.z = c.q[t * c.ld_q + shared * c.dim + n];
+        } else {
+          const int col = head * c.dim + n;
+          const float low = c.lower[col];
+          const float raw = c.g[t * c.ld_g + col] + (c.g_bias ? c.g_bias[col] : 0.f);
+          const float f = low + (1.0f - low) / (1.0f + expf(-raw));
+          in.x = f;
+          in.y = 1.0f - f;
+          in.z = silu_f(c.q[t * c.ld_q + col]);
+        }
+      }
+      gkq[e] = in;
+    }
+    for (int e = lane; e < count * 4; e += 64) {
+      const int i = e >> 2, ch = tile * 4 + (e & 3);
+      const int64_t t = t0 + i;
+      const float v = ch < c.vdim ? c.v[t * c.ld_v + head * c.vdim + ch] : 0.f;
+      const float b = FORM == 0 ? 1.0f / (1.0f + expf(-c.beta[t * c.ld_beta + head])) : 1.0f;
+      tok[e] = make_float2(v, b);
+    }
+    __syncthreads();
+    if (FORM == 0 && c.unit) {          // q and k as unit vectors: sixteen lanes take a token
+      for (int i = threadIdx.x >> 4; i < count; i += 4 * KS_WAVES) {
+        float sk = 0.f, sq = 0.f;
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+          const float4 e = gkq[i * NP + sub + 16 * r];
+          sk = fmaf(e.y, e.y, sk);
+          sq = fmaf(e.z, e.z, sq);
+        }
+        const float rk = 1.0f / sqrtf(sum_of_16_lanes(sk) + c.unit_eps);
+        const float rq = c.q_scale / sqrtf(sum_of_16_lanes(sq) + c.unit_eps);
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+          float4 e = gkq[i * NP + sub + 16 * r];
+          e.y *= rk;
+          e.z *= rq;
+          gkq[i * NP + sub + 16 * r] = e;
+        }
+      }
+      __syncthreads();
+    }
+    if (!works) continue;
+    for (int i = 0; i < count; ++i) {
+      const float2 vb = tok[i * 4 + pl];
+      float4 in[R];
+#pragma unroll
+      for (int r = 0; r < R; ++r) in[r] = gkq[i * NP + sub + 16 * r];
+      float u = vb.x;
+      if (FORM == 0) {
+        float answered = 0.f;
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+          S[r] *= in[r].x;
+          answered = fmaf(S[r], in[r].y, answered);
+        }
+        u = vb.y * (vb.x - sum_of_16_lanes(answered));
+      } else {
+#pragma unroll
+        for (int r = 0; r < R; ++r) S[r] *= in[r].x;
+      }
+      float acc = 0.f;
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        S[r] = fmaf(in[r].y, u, S[r]);
+        acc = fmaf(S[r], in[r].z, acc);
+      }
+      const float o = sum_of_16_lanes(acc);
+      if (live && sub == 0) ocol[(int64_t)(t0 + i) * c.ld_out] = o;
+    }
+  }
+  if (!works) return;
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const int n = sub + 16 * r;
+    if (n < c.dim) held[(int64_t)n * 4] = S[r];
+  }
+}
+
+template <int R>
+static void launch_keyed_scan(hipStream_t stream, const KeyedScanCall& c) {
+  const int per_token = 4 * 16 * R + 8 * KS_WAVES;
+  const int tiles = (c.vdim + 3) / 4, groups = (tiles + KS_WAVES - 1) / KS_WAVES;
+  const int chunk = scan_chunk(per_token, c.tokens);
+  dim3 grid(groups, c.heads, c.n_seqs), block(64 * KS_WAVES);
+  const size_t lds = (size_t)chunk * per_token * sizeof(float);
+  if (c.form == 0)
+    hipLaunchKernelGGL((keyed_scan_kernel<R, 0>), grid, block, lds, stream, c, chunk, tiles);
+  else
+    hipLaunchKernelGGL((keyed_scan_kernel<R, 1>), grid, block, lds, stream, c, chunk, tiles);
+}
+
+BT_EXPORT int bt_keyed_scan_call(void* stream, const KeyedScanCall* c) {
+  if (c->tokens <= 0 || c->n_seqs <= 0) return BT_OK;
+  if (c->heads <= 0 || c->dim <= 0 || c->dim > 256 || c->vdim <= 0)
+    BT_REFUSE("keyed_scan: %d heads with keys of %d (1..256) and values of %d", c->heads, c->dim, c->vdim);
+  if (c->form != 0 && c->form != 1) BT_REFUSE("keyed_scan: unknown form %d", c->form);
+  if (c->form == 0 && (c->kv_heads <= 0 || c->heads % c->kv_heads != 0))
+    BT_REFUSE("keyed_scan: %d heads cannot share %d heads of queries and keys", c->heads, c->kv_heads);
+  if (!c->q || !c->v || !c->g || !c->out || !c->S || !c->seq_off || !c->slots)
+    BT_REFUSE("keyed_scan: missing operand");
+  if (c->form == 0 && (!c->k || !c->beta || !c->A_log)) BT_REFUSE("keyed_scan: the delta rule lacks keys, beta or A_log");
+  if (c->form == 1 && !c->lower) BT_REFUSE("keyed_scan: the forget gate lacks its lower bound");
+  const int64_t qk = (int64_t)(c->form == 0 ? c->kv_heads : c->heads) * c->dim;
+  if (c->ld_q < qk || (c->form == 0 && c->ld_k < qk) || c->ld_g < (int64_t)c->heads * c->dim ||
+      c->ld_v < (int64_t)c->heads * c->vdim || c->ld_out < (int64_t)c->heads * c->vdim ||
+      (c->form == 0 && c->ld_beta < c->heads))
+    BT_REFUSE("keyed_scan: rows too short for %d heads of %d and %d", c->heads, c->dim, c->vdim);
+  if (c->state_stride < (int64_t)c->heads * ((c->vdim + 3) / 4) * c->dim * 4)
+    BT_REFUSE("keyed_scan: a slot's state of %lld elements does not hold %d heads of %d x %d", (long long)c->state_stride,
+              c->heads, c->dim, c->vdim);
+  if (c->heads > 65535 || c->n_seqs > 65535) BT_REFUSE("keyed_scan: %d heads of %d sequences are too many", c->heads, c->n_seqs);
+  hipStream_t s = (hipStream_t)stream;
+  const int per = (c->dim + 15) / 16;
+  if (per <= 1) launch_keyed_scan<1>(s, *c);
+  else if (per <= 2) launch_keyed_scan<2>(s, *c);
+  else if (per <= 4) launch_keyed_scan<4>(s, *c);
+  else if (per <= 8) launch_keyed_scan<8>(s, *c);
+  else launch_keyed_scan<16>(s, *c);
+  return bt_check_launch("keyed_scan");
+}
+
+// out[t][h * vdim + i] = y / sqrt(mean_i(y^2) + eps) * weight[i] * sigmoid(gate[t][h * vdim + i]), y = the
+// head's read-out; without `gate` no last factor.  Columns of `out` behind the heads are set to zero.
+struct HeadNormGateCall {
+  int out_dtype;          // 0 float32, 1 bfloat16
+  int tokens, heads, vdim;
+  int out_cols;           // columns of out written: heads * vdim, then zeros
+  float eps;
+  float mult;             // one more factor on the result
+  const float* y;         // [tokens][ld_y]
+  int64_t ld_y;
+  const float* gate;      // [tokens][ld_gate] logits, or null
+  int64_t ld_gate;
+  const float* weight;    // [vdim]
+  void* out;              // [tokens][ld_out]
+  int64_t ld_out;
+};
+
+template <typename T>
+__global__ void __launch_bounds__(256) head_norm_gate_kernel(HeadNormGateCall c) {
+  const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  T* out = static_cast<T*>(c.out) + (int64_t)t * c.ld_out;
+  for (int head = blockIdx.y * 4 + wave; head < c.heads; head += gridDim.y * 4) {
+    const float* y = c.y + (int64_t)t * c.ld_y + head * c.vdim;
+    float squares = 0.f;
+    for (int i = lane; i < c.vdim; i += 64) squares = fmaf(y[i], y[i], squares);
+    const float scale = c.mult / sqrtf(wave_sum(squares) / (float)c.vdim + c.eps);
+    for (int i = lane; i < c.vdim; i += 64) {
+      float v = y[i] * scale * c.weight[i];
+      if (c.gate) v *= 1.0f / (1.0f + expf(-c.gate[(int64_t)t * c.ld_gate + head * c.vdim + i]));
+      out[head * c.vdim + i] = from_float<T>(v);
+    }
+  }
+  if (blockIdx.y == 0)
+    for (int col = c.heads * c.vdim + threadIdx.x; col < c.out_cols; col += blockDim.x) out[col] = from_float<T>(0.f);
+}
+
+BT_EXPORT int bt_head_norm_gate_call(void* stream, const HeadNormGateCall* c) {
+  if (c->tokens <= 0) return BT_OK;
+  if (c->heads <= 0 || c->vdim <= 0) BT_REFUSE("head_norm_gate: %d heads of %d", c->heads, c->vdim);
+  const int64_t columns = (int64_t)c->heads * c->vdim;
+  if (!c->y || !c->weight || !c->out || c->ld_y < columns || c->out_cols < columns || c->ld_out < c->out_cols ||
+      (c->gate && c->ld_gate < columns))
+    BT_REFUSE("head_norm_gate: missing operand or rows too short");
+  int per_token = (c->heads + 3) / 4;
+  if (per_token > 64) per_token = 64;
+  dim3 grid(c->tokens, per_token), block(256);
+  if (c->out_dtype == 0)
+    hipLaunchKernelGGL(head_norm_gate_kernel<float>, grid, block, 0, (hipStream_t)stream, *c);
+  else
+    hipLaunchKernelGGL(head_norm_gate_kernel<bf16_t>, grid, block, 0, (hipStream_t)stream, *c);
+  return bt_check_launch("head_norm_gate");
+}

@@ -5,8 +5,11 @@
 //     position, queries go to a buffer for the attention kernel and keys and values straight into
 //     the paged cache at the token's position.  Queries/keys and values may have different head
 //     sizes; the cache keeps heads of one size, and what lies behind a head's own channels is zero.
-// Channel i < rot_dims / 2 is paired with channel i + rot_dims / 2; the pair (u, v) at position p
-// becomes (u cos a - v sin a, v cos a + u sin a), a = p * inv_freq[i].  The frequencies come as a
+// Channel i < rot_dims / 2 is paired with channel i + rot_dims / 2 (`pairing` 0, the halves) or channel
+// 2 i with channel 2 i + 1 (`pairing` 1, neighbours); the pair (u, v) at position p
+// becomes (u cos a - v sin a, v cos a + u sin a), a = p * inv_freq[i].  With `norm_span` 1 the root mean
+// square is taken over a token's WHOLE query (or key) projection, all heads at once, and the scale has
+// an entry for every channel of the projection.  The frequencies come as a
 // table, so any schedule of them (scaled, interpolated) is the caller's.  Norms, angles and the
 // rotation are 32-bit.
 #include "host.h"
@@ -20,14 +23,16 @@ struct HeadRotaryCall {
   float eps;
   const float* in;        // [tokens][ld] float32: queries (heads * dim), keys (kv_heads * dim), values (kv_heads * vdim)
   int64_t ld;
-  const float* q_gamma;   // [dim] or null: no norm of the query heads
-  const float* k_gamma;   // [dim] or null
+  const float* q_gamma;   // [dim] ([heads * dim] with norm_span 1) or null: no norm of the queries
+  const float* k_gamma;   // [dim] ([kv_heads * dim] with norm_span 1) or null
   const float* inv_freq;  // [rot_dims / 2]
   void* q_out;            // [tokens][ld_q]: head j at columns j * kv.head_dim
   int64_t ld_q;
   const int* tok_seq;
   const int* tok_pos;
   KvView kv;              // kv_heads heads of head_dim >= max(dim, vdim)
+  int pairing;            // 0: channel i turns with channel i + rot_dims / 2; 1: channel 2 i with channel 2 i + 1
+  int norm_span;          // 0: every head over its own root mean square; 1: the whole projection over one
 };
 
 #define HR_WAVES 4
@@ -57,7 +62,15 @@ __global__ void __launch_bounds__(HR_WAVES * 64) head_rotary_kernel(HeadRotaryCa
       row[col] = v;
       squares += v * v;
     }
-    if (gamma) {
+    if (gamma && c.norm_span == 1) {
+      // every wave of a projection adds up the same squares in the same order: the heads agree exactly
+      const int all = (is_q ? c.heads : c.kv_heads) * c.dim;
+      const float* whole = c.in + (int64_t)t * c.ld + (is_q ? 0 : (int64_t)c.heads * c.dim);
+      squares = 0.f;
+      for (int col = lane; col < all; col += 64) squares = fmaf(whole[col], whole[col], squares);
+      const float rstd = 1.0f / sqrtf(wave_sum(squares) / (float)all + c.eps);
+      for (int col = lane; col < n; col += 64) row[col] = row[col] * rstd * gamma[head * c.dim + col];
+    } else if (gamma) {
       const float rstd = 1.0f / sqrtf(wave_sum(squares) / (float)n + c.eps);
       for (int col = lane; col < n; col += 64) row[col] = row[col] * rstd * gamma[col];
     }
@@ -88,9 +101,10 @@ __global__ void __launch_bounds__(HR_WAVES * 64) head_rotary_kernel(HeadRotaryCa
     for (int i = lane; i < half; i += 64) {
       float sn, cs;
       sincosf((float)pos * c.inv_freq[i], &sn, &cs);
-      const float u = row[i], v = row[i + half];
-      store(i, u * cs - v * sn);
-      store(i + half, v * cs + u * sn);
+      const int first = c.pairing == 1 ? 2 * i : i, second = c.pairing == 1 ? 2 * i + 1 : i + half;
+      const float u = row[first], v = row[second];
+      store(first, u * cs - v * sn);
+      store(second, v * cs + u * sn);
     }
   for (int col = (turned ? c.rot_dims : 0) + lane; col < hd; col += 64) store(col, col < n ? row[col] : 0.f);
 }
@@ -101,6 +115,8 @@ BT_EXPORT int bt_head_rotary_call(void* stream, const HeadRotaryCall* c) {
     BT_REFUSE("head_rotary: %d query heads cannot share %d key/value heads", c->heads, c->kv_heads);
   if (c->dim <= 0 || c->vdim <= 0 || c->dim > HR_MAX_DIM || c->vdim > HR_MAX_DIM)
     BT_REFUSE("head_rotary: head sizes %d and %d outside 1..%d", c->dim, c->vdim, HR_MAX_DIM);
+  if ((c->pairing != 0 && c->pairing != 1) || (c->norm_span != 0 && c->norm_span != 1))
+    BT_REFUSE("head_rotary: pairing %d and norm_span %d must be 0 or 1", c->pairing, c->norm_span);
   if (c->rot_dims < 0 || c->rot_dims % 2 != 0 || c->rot_dims > c->dim)
     BT_REFUSE("head_rotary: %d turned channels must be even and at most the head size %d", c->rot_dims, c->dim);
   if (c->kv.kv_heads != c->kv_heads || c->kv.head_dim < c->dim || c->kv.head_dim < c->vdim || c->kv.head_dim > HR_MAX_DIM)

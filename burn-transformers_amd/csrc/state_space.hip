@@ -8,6 +8,7 @@
 //   * scan with one decay per head and a state of [state, head size] (state-space duality form)
 //   * gate, then RMS norm in equal parts
 #include "host.h"
+#include "scan.h"
 
 
 // Brings rows t0 .. t0 + count - 1 of B and C (`state` columns each, row pitch `ld`, 32-bit offsets) into LDS
@@ -56,30 +57,6 @@ __device__ __forceinline__ void fill_pairs(float2* BC, const float* B, const flo
     fill_pairs_ahead<NP, 2048 / THREADS, THREADS>(BC, B, C, ld, t0, count, state, lane);
 }
 
-// Sums over groups of 8 or 16 neighbouring lanes with data-parallel moves between lanes of a row
-// (no trip through the LDS crossbar as a shuffle takes; a recurrence pays this once per token): first
-// within quads (swap neighbours, swap pairs: then every lane of a quad holds the quad's sum), then
-// the mirror image within half a row pairs the two quads of eight lanes, then the mirror image within
-// the row pairs its halves.  Every lane of the group ends with the group's sum.
-template <int CTRL>
-__device__ __forceinline__ float dpp_move(float v) {
-  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false));
-}
-__device__ __forceinline__ float sum_of_8_lanes(float v) {
-  v += dpp_move<0xB1>(v);     // quad_perm [1, 0, 3, 2]
-  v += dpp_move<0x4E>(v);     // quad_perm [2, 3, 0, 1]
-  v += dpp_move<0x141>(v);    // row_half_mirror
-  return v;
-}
-__device__ __forceinline__ float sum_of_16_lanes(float v) {
-  v = sum_of_8_lanes(v);
-  v += dpp_move<0x140>(v);    // row_mirror
-  return v;
-}
-
-__device__ __forceinline__ float silu_f(float v) { return v / (1.0f + expf(-v)); }
-__device__ __forceinline__ float softplus_f(float v) { return v > 20.0f ? v : log1pf(expf(v)); }
-
 // ---------------------------------------------------------------------------------------------
 struct CausalConvCall {
   int cast_dtype;         // element type of `cast`
@@ -88,7 +65,7 @@ struct CausalConvCall {
   const float* in;        // [tokens][ld_in]
   int64_t ld_in;
   const float* weight;    // [channels][taps]; the last tap meets the current token
-  const float* bias;      // [channels]
+  const float* bias;      // [channels], or null: none
   float* out;             // [tokens][ld_out] float32
   int64_t ld_out;
   void* cast;             // [tokens][ld_cast] the same in the products' type, or null
@@ -114,7 +91,7 @@ __global__ void __launch_bounds__(256) causal_conv_kernel(CausalConvCall c) {
   const int seq = c.tok_seq[t];
   const int local = t - c.seq_off[seq];
   float* held = c.state + (int64_t)c.slots[seq] * c.state_stride;
-  float sum = c.bias[ch];
+  float sum = c.bias ? c.bias[ch] : 0.f;
   for (int j = 0; j < c.taps; ++j) {
     const int back = c.taps - 1 - j;
     const int src = local - back;
@@ -150,7 +127,7 @@ BT_EXPORT int bt_causal_conv_call(void* stream, const CausalConvCall* c) {
   if (c->tokens <= 0) return BT_OK;
   if (c->channels <= 0 || c->taps <= 0 || c->n_seqs <= 0)
     BT_REFUSE("causal_conv: %d channels, %d taps, %d sequences: all must be positive", c->channels, c->taps, c->n_seqs);
-  if (!c->in || !c->weight || !c->bias || !c->out || !c->tok_seq || !c->seq_off || !c->slots || (c->taps > 1 && !c->state))
+  if (!c->in || !c->weight || !c->out || !c->tok_seq || !c->seq_off || !c->slots || (c->taps > 1 && !c->state))
     BT_REFUSE("causal_conv: missing operand");
   if (c->ld_in < c->channels || c->ld_out < c->channels || (c->cast && (c->cast_cols < c->channels || c->ld_cast < c->cast_cols)))
     BT_REFUSE("causal_conv: the rows do not hold %d channels", c->channels);
@@ -177,16 +154,18 @@ BT_EXPORT int bt_causal_conv_call(void* stream, const CausalConvCall* c) {
 }
 
 // ---------------------------------------------------------------------------------------------
-// out[t][c] = softplus(sum_r W[c][r] * low[t][r] + bias[c]); the rank is small.
+// out[t][c] = act(sum_r W[c][r] * low[t][r] + bias[c]), act the softplus (`act` 0), the sigmoid (1) or
+// nothing (2); the rank is small.
 struct DtProjectCall {
   int dtype;              // element type of W
   int tokens, channels, rank;
   const float* low;       // [tokens][ld_low]
   int64_t ld_low;
   const void* W;          // [channels][rank]
-  const float* bias;      // [channels]
+  const float* bias;      // [channels], or null: none
   float* out;             // [tokens][ld_out]
   int64_t ld_out;
+  int act;                // 0: softplus, 1: sigmoid, 2: none
 };
 
 // TOKENS tokens share a work-group (their rows of `low` wait in LDS, every weight is read once for
@@ -213,10 +192,13 @@ __global__ void __launch_bounds__(256) dt_project_kernel(DtProjectCall c) {
 #pragma unroll
     for (int i = 0; i < TOKENS; ++i) acc[i] = fmaf(wv, rows[i * c.rank + r], acc[i]);
   }
-  const float b = c.bias[ch];
+  const float b = c.bias ? c.bias[ch] : 0.f;
 #pragma unroll
   for (int i = 0; i < TOKENS; ++i)
-    if (t0 + i < c.tokens) c.out[(int64_t)(t0 + i) * c.ld_out + ch] = softplus_f(acc[i] + b);
+    if (t0 + i < c.tokens) {
+      const float z = acc[i] + b;
+      c.out[(int64_t)(t0 + i) * c.ld_out + ch] = c.act == 0 ? softplus_f(z) : (c.act == 1 ? 1.0f / (1.0f + expf(-z)) : z);
+    }
 }
 
 template <typename T, int TOKENS>
@@ -229,8 +211,9 @@ BT_EXPORT int bt_dt_project_call(void* stream, const DtProjectCall* c) {
   if (c->tokens <= 0) return BT_OK;
   if (c->channels <= 0 || c->rank <= 0 || c->rank > 1024)
     BT_REFUSE("dt_project: %d channels from rank %d (1..1024)", c->channels, c->rank);
-  if (!c->low || !c->W || !c->bias || !c->out || c->ld_low < c->rank || c->ld_out < c->channels)
+  if (!c->low || !c->W || !c->out || c->ld_low < c->rank || c->ld_out < c->channels)
     BT_REFUSE("dt_project: missing operand or rows too short");
+  if (c->act < 0 || c->act > 2) BT_REFUSE("dt_project: unknown activation %d", c->act);
   hipStream_t s = (hipStream_t)stream;
   if (c->tokens <= 16) {
     if (c->dtype == 0) launch_dt_project<float, 1>(s, *c);
@@ -417,13 +400,6 @@ __global__ void __launch_bounds__(64) selective_scan_kernel(SelectiveScanCall c,
   if (blockIdx.x == 0)
     for (int t = first; t < last; ++t)
       for (int col = c.channels + lane; col < c.out_cols; col += 64) out[(int64_t)t * c.ld_out + col] = from_float<T>(0.f);
-}
-
-// Tokens of a run: as many as keep a work-group's LDS at about 24 KiB, at most 64, no more than the step has.
-static int scan_chunk(int floats_per_token, int tokens) {
-  int chunk = 6144 / floats_per_token;
-  chunk = chunk < 1 ? 1 : chunk > 64 ? 64 : chunk;
-  return chunk < tokens ? chunk : tokens;
 }
 
 // C_k = exp(A * sum of dt of span k) * C_(k-1) + E_k along every sequence, in place; C_(-1), the state the

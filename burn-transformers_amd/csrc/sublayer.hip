@@ -360,3 +360,134 @@ BT_EXPORT int bt_poly_norm_call(void* stream, const PolyNormCall* c) {
     hipLaunchKernelGGL(poly_norm_kernel<bf16_t>, grid, block, lds, (hipStream_t)stream, *c);
   return bt_check_launch("poly_norm");
 }
+
+// RMS norm in equal consecutive parts of a row ("groups"), each over its own root mean square, the whole
+// times `gamma`; of a sublayer's output on its way into the stream, or of rows of the stream itself.
+//   output (n_delta > 0):  v = scale * (sum of delta + bias) + scale2 * (sum of delta2 + bias2), the second
+//       term for layers whose sublayer is two parts side by side; v *= sigmoid(gate) where a gate's
+//       logits come with it; x[t] (+)= mult * N(v), and `cast` receives the new x in the products' type.
+//   rows (n_delta == 0):   cast[r] = N(x[rows[r]]) (every row in order without `rows`); x stays as it is.
+struct GroupNormCall {
+  int cast_dtype;         // element type of `cast`: 0 float32, 1 bfloat16
+  int tokens;             // rows of this call
+  int width;
+  int groups;             // equal parts of a row, each with statistics of its own
+  int n_delta, n_delta2;
+  int accumulate;         // output: 1: x += mult * N(v); 0: x = mult * N(v)
+  int cast_cols;          // columns of `cast` that are written: the result, then zeros
+  float eps, mult;
+  float scale, scale2;    // factors of the two terms
+  float* x;               // [..][width] float32 residual stream
+  const float* delta;     // [n_delta][..][ldd]
+  int64_t delta_stride, ldd;
+  const float* bias;      // [width] or null
+  const float* delta2;    // [n_delta2][..][ldd2], or null
+  int64_t delta2_stride, ldd2;
+  const float* bias2;     // [width] or null
+  const float* gate;      // [tokens][ld_gate] logits, or null
+  int64_t ld_gate;
+  const float* gamma;     // [width]
+  void* cast;             // [tokens][ld_cast], or null
+  int64_t ld_cast;
+  const int* rows;        // rows mode: which rows of x, or null
+};
+
+template <typename T>
+__global__ void __launch_bounds__(256) group_norm_kernel(GroupNormCall c) {
+  extern __shared__ float row_buf[];          // [width], then [groups] reciprocal roots
+  float* rstd = row_buf + c.width;
+  const int t = blockIdx.x;
+  const bool from_stream = c.n_delta == 0;
+  const int source = from_stream && c.rows ? c.rows[t] : t;
+  float* xr = c.x + (int64_t)source * c.width;
+  for (int col = threadIdx.x; col < c.width; col += blockDim.x) {
+    float v;
+    if (from_stream) {
+      v = xr[col];
+    } else {
+      v = c.bias ? c.bias[col] : 0.f;
+      for (int s = 0; s < c.n_delta; ++s) v += c.delta[s * c.delta_stride + (int64_t)t * c.ldd + col];
+      v *= c.scale;
+      if (c.n_delta2 > 0) {
+        float w = c.bias2 ? c.bias2[col] : 0.f;
+        for (int s = 0; s < c.n_delta2; ++s) w += c.delta2[s * c.delta2_stride + (int64_t)t * c.ldd2 + col];
+        v = fmaf(c.scale2, w, v);
+      }
+      if (c.gate) v *= 1.0f / (1.0f + expf(-c.gate[(int64_t)t * c.ld_gate + col]));
+    }
+    row_buf[col] = v;
+  }
+  __syncthreads();
+  // a wave takes whole parts, so no sum crosses waves
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = blockDim.x >> 6;
+  const int per = c.width / c.groups;
+  for (int g = wave; g < c.groups; g += waves) {
+    float squares = 0.f;
+    for (int i = lane; i < per; i += 64) squares = fmaf(row_buf[g * per + i], row_buf[g * per + i], squares);
+    squares = wave_sum(squares);
+    if (lane == 0) rstd[g] = 1.0f / sqrtf(squares / (float)per + c.eps);
+  }
+  __syncthreads();
+  T* cast = static_cast<T*>(c.cast);
+  for (int col = threadIdx.x; col < c.width; col += blockDim.x) {
+    float y = row_buf[col] * rstd[col / per] * c.gamma[col];
+    if (!from_stream) {
+      y *= c.mult;
+      if (c.accumulate) y += xr[col];
+      xr[col] = y;
+    }
+    if (cast) cast[(int64_t)t * c.ld_cast + col] = from_float<T>(y);
+  }
+  if (cast)
+    for (int col = c.width + threadIdx.x; col < c.cast_cols; col += blockDim.x)
+      cast[(int64_t)t * c.ld_cast + col] = from_float<T>(0.f);
+}
+
+BT_EXPORT int bt_group_norm_call(void* stream, const GroupNormCall* c) {
+  if (c->tokens <= 0) return BT_OK;
+  if (c->width <= 0 || c->width > 15360) BT_REFUSE("group_norm: width %d outside 1..15360", c->width);
+  if (c->groups <= 0 || c->groups > 512 || c->width % c->groups != 0)
+    BT_REFUSE("group_norm: %d parts (1..512) must divide width %d", c->groups, c->width);
+  if (!c->x || !c->gamma || (c->n_delta > 0 && !c->delta) || (c->n_delta2 > 0 && !c->delta2))
+    BT_REFUSE("group_norm: missing operand");
+  if (c->n_delta == 0 && (!c->cast || c->n_delta2 > 0 || c->gate))
+    BT_REFUSE("group_norm: rows of the stream are normalised into `cast`, with one term and no gate");
+  if (c->n_delta < 0 || c->n_delta2 < 0) BT_REFUSE("group_norm: negative counts of partial sums");
+  if (c->cast && (c->cast_cols < c->width || c->ld_cast < c->cast_cols))
+    BT_REFUSE("group_norm: a copy of %d columns in rows of %lld does not hold width %d", c->cast_cols,
+              (long long)c->ld_cast, c->width);
+  if (c->gate && c->ld_gate < c->width) BT_REFUSE("group_norm: the gate's rows are shorter than the width");
+  const size_t lds = (size_t)(c->width + c->groups) * sizeof(float);
+  dim3 grid(c->tokens), block(256);
+  if (c->cast_dtype == 0)
+    hipLaunchKernelGGL(group_norm_kernel<float>, grid, block, lds, (hipStream_t)stream, *c);
+  else
+    hipLaunchKernelGGL(group_norm_kernel<bf16_t>, grid, block, lds, (hipStream_t)stream, *c);
+  return bt_check_launch("group_norm");
+}
+
+// logits <- cap * tanh(logits / cap), in place, over float32 rows.
+struct SoftCapCall {
+  int rows;
+  int columns;
+  float cap;
+  float* logits;          // [rows][ld]
+  int64_t ld;
+};
+
+__global__ void __launch_bounds__(256) soft_cap_kernel(SoftCapCall c) {
+  float* row = c.logits + (int64_t)blockIdx.x * c.ld;
+  const float inverse = 1.0f / c.cap;
+  for (int col = blockIdx.y * blockDim.x + threadIdx.x; col < c.columns; col += gridDim.y * blockDim.x)
+    row[col] = c.cap * tanhf(row[col] * inverse);
+}
+
+BT_EXPORT int bt_soft_cap_call(void* stream, const SoftCapCall* c) {
+  if (c->rows <= 0) return BT_OK;
+  if (c->columns <= 0 || c->ld < c->columns || !c->logits) BT_REFUSE("soft_cap: missing operand or rows too short");
+  if (!(c->cap > 0.f)) BT_REFUSE("soft_cap: the cap %g must be positive", (double)c->cap);
+  int per_row = (c->columns + 2047) / 2048;
+  if (per_row > 64) per_row = 64;
+  hipLaunchKernelGGL(soft_cap_kernel, dim3(c->rows, per_row), dim3(256), 0, (hipStream_t)stream, *c);
+  return bt_check_launch("soft_cap");
+}

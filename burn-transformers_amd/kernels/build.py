@@ -87,7 +87,7 @@ def entry_points(name):
 
 
 # the package's own modules
-for _name in ("core", "gemm_mfma", "attention_f32", "sublayer", "latent", "state_space", "rotary", "experts"):
+for _name in ("core", "gemm_mfma", "attention_f32", "sublayer", "latent", "state_space", "rotary", "experts", "linear_attention"):
     register_module(_name, _name + ".hip", _own=True)
 register_module("gemm_library", "gemm_library.hip", ["-ldl"], _own=True)   # host code around hipBLASLt, opened at run time
 register_module("program", "program.cpp", _own=True)                       # the host loop that walks a launch list

@@ -48,7 +48,7 @@ class AttnArgs(ctypes.Structure):
                 ("tok_seq", _c_ptr), ("tok_pos", _c_ptr), ("seq_off", _c_ptr), ("seq_start", _c_ptr),
                 ("kv", KvView), ("q_heads", _c_int), ("n_tokens", _c_int), ("n_seqs", _c_int),
                 ("max_count", _c_int), ("window", _c_int), ("scale", _c_float), ("splits", _c_int),
-                ("partial", _c_ptr), ("out_rows", _c_int), ("chunk", _c_int)]
+                ("partial", _c_ptr), ("out_rows", _c_int), ("chunk", _c_int), ("sink", _c_ptr)]
 
 
 class NormOperand(ctypes.Structure):
@@ -58,7 +58,8 @@ class NormOperand(ctypes.Structure):
 
 class EmbedCall(ctypes.Structure):
     _fields_ = [("dtype", _c_int), ("tokens", _c_int), ("width", _c_int), ("ids", _c_ptr), ("pos", _c_ptr),
-                ("table", _c_ptr), ("positions", _c_ptr), ("out", _c_ptr), ("scale", _c_float), ("copy", _c_ptr)]
+                ("table", _c_ptr), ("positions", _c_ptr), ("out", _c_ptr), ("scale", _c_float), ("copy", _c_ptr),
+                ("cast", _c_ptr), ("cast_cols", _c_int)]
 
 
 class AddNormCall(ctypes.Structure):
@@ -130,7 +131,7 @@ class CausalConvCall(ctypes.Structure):
 
 class DtProjectCall(ctypes.Structure):
     _fields_ = [("dtype", _c_int), ("tokens", _c_int), ("channels", _c_int), ("rank", _c_int), ("low", _c_ptr),
-                ("ld_low", _c_i64), ("W", _c_ptr), ("bias", _c_ptr), ("out", _c_ptr), ("ld_out", _c_i64)]
+                ("ld_low", _c_i64), ("W", _c_ptr), ("bias", _c_ptr), ("out", _c_ptr), ("ld_out", _c_i64), ("act", _c_int)]
     _step_fields_ = {"tokens": "tokens"}
 
 
@@ -163,14 +164,15 @@ class HeadRotaryCall(ctypes.Structure):
     _fields_ = [("dtype", _c_int), ("tokens", _c_int), ("heads", _c_int), ("kv_heads", _c_int), ("dim", _c_int),
                 ("vdim", _c_int), ("rot_dims", _c_int), ("eps", _c_float), ("input", _c_ptr), ("ld", _c_i64),
                 ("q_gamma", _c_ptr), ("k_gamma", _c_ptr), ("inv_freq", _c_ptr), ("q_out", _c_ptr), ("ld_q", _c_i64),
-                ("tok_seq", _c_ptr), ("tok_pos", _c_ptr), ("kv", KvView)]
+                ("tok_seq", _c_ptr), ("tok_pos", _c_ptr), ("kv", KvView), ("pairing", _c_int), ("norm_span", _c_int)]
     _step_fields_ = {"tokens": "tokens"}
 
 
 class RouteCall(ctypes.Structure):
     _fields_ = [("dtype", _c_int), ("tokens", _c_int), ("width", _c_int), ("experts", _c_int), ("top", _c_int),
                 ("groups", _c_int), ("keep", _c_int), ("h", _c_ptr), ("ldh", _c_i64), ("W", _c_ptr),
-                ("correction", _c_ptr), ("gate_w", _c_ptr), ("weights", _c_ptr), ("gate", _c_ptr)]
+                ("correction", _c_ptr), ("gate_w", _c_ptr), ("weights", _c_ptr), ("gate", _c_ptr), ("score", _c_int),
+                ("group_rank", _c_int), ("normalize", _c_int)]
     _step_fields_ = {"tokens": "tokens"}
 
 
@@ -178,7 +180,38 @@ class GatedExpertsCall(ctypes.Structure):
     _fields_ = [("dtype", _c_int), ("tokens", _c_int), ("experts", _c_int), ("ff", _c_int), ("shared_ff", _c_int),
                 ("identity", _c_int), ("hidden_cols", _c_int), ("width", _c_int), ("gu", _c_ptr), ("ld_gu", _c_i64),
                 ("weights", _c_ptr), ("gate", _c_ptr), ("hidden", _c_ptr), ("ld_hidden", _c_i64), ("h", _c_ptr),
-                ("ldh", _c_i64), ("identity_out", _c_ptr)]
+                ("ldh", _c_i64), ("identity_out", _c_ptr), ("act", _c_int), ("limit", _c_float), ("alpha", _c_float)]
+    _step_fields_ = {"tokens": "tokens"}
+
+
+class GroupNormCall(ctypes.Structure):
+    _fields_ = [("cast_dtype", _c_int), ("tokens", _c_int), ("width", _c_int), ("groups", _c_int), ("n_delta", _c_int),
+                ("n_delta2", _c_int), ("accumulate", _c_int), ("cast_cols", _c_int), ("eps", _c_float), ("mult", _c_float),
+                ("scale", _c_float), ("scale2", _c_float), ("x", _c_ptr), ("delta", _c_ptr), ("delta_stride", _c_i64),
+                ("ldd", _c_i64), ("bias", _c_ptr), ("delta2", _c_ptr), ("delta2_stride", _c_i64), ("ldd2", _c_i64),
+                ("bias2", _c_ptr), ("gate", _c_ptr), ("ld_gate", _c_i64), ("gamma", _c_ptr), ("cast", _c_ptr),
+                ("ld_cast", _c_i64), ("rows", _c_ptr)]
+
+
+class SoftCapCall(ctypes.Structure):
+    _fields_ = [("rows", _c_int), ("columns", _c_int), ("cap", _c_float), ("logits", _c_ptr), ("ld", _c_i64)]
+    _step_fields_ = {}            # its rows are the step's wanted rows, which every step of a list shares
+
+
+class KeyedScanCall(ctypes.Structure):
+    _fields_ = [("tokens", _c_int), ("n_seqs", _c_int), ("heads", _c_int), ("kv_heads", _c_int), ("dim", _c_int),
+                ("vdim", _c_int), ("form", _c_int), ("unit", _c_int), ("unit_eps", _c_float), ("q_scale", _c_float),
+                ("q", _c_ptr), ("ld_q", _c_i64), ("k", _c_ptr), ("ld_k", _c_i64), ("v", _c_ptr), ("ld_v", _c_i64),
+                ("g", _c_ptr), ("ld_g", _c_i64), ("beta", _c_ptr), ("ld_beta", _c_i64), ("A_log", _c_ptr),
+                ("g_bias", _c_ptr), ("lower", _c_ptr), ("out", _c_ptr), ("ld_out", _c_i64), ("S", _c_ptr),
+                ("state_stride", _c_i64), ("seq_off", _c_ptr), ("slots", _c_ptr)]
+    _step_fields_ = {"tokens": "tokens"}
+
+
+class HeadNormGateCall(ctypes.Structure):
+    _fields_ = [("out_dtype", _c_int), ("tokens", _c_int), ("heads", _c_int), ("vdim", _c_int), ("out_cols", _c_int),
+                ("eps", _c_float), ("mult", _c_float), ("y", _c_ptr), ("ld_y", _c_i64), ("gate", _c_ptr),
+                ("ld_gate", _c_i64), ("weight", _c_ptr), ("out", _c_ptr), ("ld_out", _c_i64)]
     _step_fields_ = {"tokens": "tokens"}
 
 
@@ -346,6 +379,8 @@ def _step_fields(call):
         return (("tokens", "tokens"),)
     if kind is AttentionCall:
         return (("args.n_tokens", "tokens"), ("args.max_count", "max_count"))
+    if kind is GroupNormCall:
+        return () if call.n_delta == 0 and call.rows else (("tokens", "tokens"),)      # (as for AddNormCall)
     declared = getattr(kind, "_step_fields_", None)
     return None if declared is None else tuple(declared.items())
 
@@ -623,13 +658,16 @@ def epilogue_qkv(q_out, n_q, n_kv, kv_view, tok_seq, tok_pos, bias=None):
 
 # --- kernels ---------------------------------------------------------------------------------
 
-def embed(ids, positions, table, position_table, out, scale=1.0, copy=None):
+def embed(ids, positions, table, position_table, out, scale=1.0, copy=None, cast=None):
     """out[t] = scale * table[ids[t]] (+ position_table[positions[t]]); out is the float32 stream,
-    ``copy`` an optional second float32 place for the same rows."""
+    ``copy`` an optional second float32 place for the same rows, ``cast`` an optional contiguous place for them in
+    the table's type (zeros behind the width), for parts that multiply by the stream itself."""
+    if cast is not None and (cast.dtype != table.dtype or not cast.is_contiguous()):
+        raise KernelError("embed: the stream's copy is contiguous and of the table's type")
     _launch(_module("core"), "bt_embed_call",
             EmbedCall(dtype=DTYPE_CODES[table.dtype], tokens=ids.numel(), width=table.shape[1], ids=ids.data_ptr(),
                       pos=_ptr(positions), table=table.data_ptr(), positions=_ptr(position_table), out=out.data_ptr(),
-                      scale=scale, copy=_ptr(copy)))
+                      scale=scale, copy=_ptr(copy), cast=_ptr(cast), cast_cols=cast.shape[1] if cast is not None else 0))
 
 
 def add_norm(x, out, gamma, beta, eps, kind="layer_norm", delta=None, bias=None, rows=None,
@@ -866,14 +904,18 @@ def _library_has_algorithm(lda, m, n, k, epilogue):
 
 
 def attention_args(q, out, kv_view, tok_seq, tok_pos, seq_off, seq_start, q_heads, n_seqs, max_count,
-                   scale, window=0, partial=None, runs=None, chunk=0):
+                   scale, window=0, partial=None, runs=None, chunk=0, sink=None):
     """``partial``: float32 [rows * q_heads * runs, head_dim + 2] for a step whose keys are cut into
     runs that separate work-groups take.  Decode steps (long contexts in small batches): rows are
     the sequences, and ``runs`` follows from the shape.  Prompt steps (few query tiles behind a long
     context): rows are the step's tokens, the buffer may be longer than this step needs, and
     ``runs`` is given.  ``out`` may be a :class:`Chunked` for the bfloat16 decode kernels.
     ``chunk`` > 0: a query at position p sees only the keys from p - p % chunk on (chunks are counted
-    from position 0 of its sequence); ``window`` > 0: only the last ``window`` positions."""
+    from position 0 of its sequence); ``window`` > 0: only the last ``window`` positions.  ``sink``: float32
+    [q_heads], a logit per head whose exponential stands in every softmax's denominator beside the keys'
+    (no key, no value, not scaled)."""
+    if sink is not None and (sink.dtype != torch.float32 or sink.numel() != q_heads or not sink.is_contiguous()):
+        raise KernelError(f"attention: the sink is one float32 logit per query head, got {tuple(sink.shape)} {sink.dtype}")
     splits = 1
     if partial is not None:
         rows = n_seqs if runs is None else q.shape[0]
@@ -886,7 +928,7 @@ def attention_args(q, out, kv_view, tok_seq, tok_pos, seq_off, seq_start, q_head
                     q=q.data_ptr(), ldq=q.stride(0), out=out.data_ptr(), ldo=out.stride(0), out_rows=_out_rows(out),
                     tok_seq=tok_seq.data_ptr(), tok_pos=tok_pos.data_ptr(), seq_off=seq_off.data_ptr(),
                     seq_start=seq_start.data_ptr(), kv=kv_view, q_heads=q_heads, n_tokens=q.shape[0],
-                    n_seqs=n_seqs, max_count=max_count, window=window or 0, scale=scale, chunk=chunk or 0)
+                    n_seqs=n_seqs, max_count=max_count, window=window or 0, scale=scale, chunk=chunk or 0, sink=_ptr(sink))
 
 
 def attention(args, dtype, decode, impl="auto"):
@@ -1091,19 +1133,22 @@ def causal_conv(rows, weight, bias, out, state, step, cast=None):
             CausalConvCall(cast_dtype=DTYPE_CODES[cast.dtype] if cast is not None else FLOAT32, tokens=rows.shape[0],
                            n_seqs=step.n_seqs, channels=channels, taps=taps,
                            cast_cols=cast.shape[1] if cast is not None else 0, input=rows.data_ptr(),
-                           ld_in=rows.stride(0), weight=weight.data_ptr(), bias=bias.data_ptr(), out=out.data_ptr(),
+                           ld_in=rows.stride(0), weight=weight.data_ptr(), bias=_ptr(bias), out=out.data_ptr(),
                            ld_out=out.stride(0), cast=_ptr(cast), ld_cast=cast.stride(0) if cast is not None else 0,
                            state=state.data_ptr(), state_stride=state.stride(0), tok_seq=step.tok_seq.data_ptr(),
                            seq_off=step.seq_off.data_ptr(), slots=step.slots.data_ptr()))
 
 
-def dt_project(low, weight, bias, out):
-    """out = softplus(low . weight^T + bias) in float32; ``low`` float32 [tokens, rank] (rows may be
-    strided), ``weight`` [channels, rank]."""
+LOW_RANK_ACTS = {"softplus": 0, "sigmoid": 1, "none": 2}
+
+
+def dt_project(low, weight, bias, out, act="softplus"):
+    """out = act(low . weight^T + bias) in float32; ``low`` float32 [tokens, rank] (rows may be
+    strided), ``weight`` [channels, rank], ``bias`` [channels] or None, ``act`` "softplus", "sigmoid" or "none"."""
     _launch(_module("state_space"), "bt_dt_project_call",
             DtProjectCall(dtype=DTYPE_CODES[weight.dtype], tokens=low.shape[0], channels=weight.shape[0],
                           rank=weight.shape[1], low=low.data_ptr(), ld_low=low.stride(0), W=weight.data_ptr(),
-                          bias=bias.data_ptr(), out=out.data_ptr(), ld_out=out.stride(0)))
+                          bias=_ptr(bias), out=out.data_ptr(), ld_out=out.stride(0), act=LOW_RANK_ACTS[act]))
 
 
 SCAN_SPAN = 64        # tokens of a span of a long sequence (sequences of three spans or more are cut); 0: never cut
@@ -1162,42 +1207,122 @@ def gated_norm(y, z, weight, parts, eps, out):
 # --- rotary positions -------------------------------------------------------------------------
 
 def head_rotary(fused, heads, kv_heads, dim, vdim, rot_dims, inv_freq, q_gamma, k_gamma, eps, q_out, tok_seq, tok_pos,
-                kv_view, dtype):
+                kv_view, dtype, neighbours=False, whole_norm=False):
     """Behind a fused query/key/value projection with float32 rows ``fused`` (queries heads * dim, keys
     kv_heads * dim, values kv_heads * vdim): every query and key head divided by its root mean square
     times ``q_gamma`` / ``k_gamma`` ([dim] float32; None: no norm), the first ``rot_dims`` channels of each
     turned by the token's position (channel i with i + rot_dims / 2, angle position * ``inv_freq[i]``);
     queries go to ``q_out`` (head j at columns j * head size of the cache, zeros behind its own
-    channels), keys and values into the paged cache at each token's position."""
+    channels), keys and values into the paged cache at each token's position.
+    ``neighbours``: channel 2 i turns with channel 2 i + 1 instead.  ``whole_norm``: the root mean square is
+    taken over the token's whole query (key) projection and the scales are [heads * dim] ([kv_heads * dim])."""
     _launch(_module("rotary"), "bt_head_rotary_call",
             HeadRotaryCall(dtype=DTYPE_CODES[dtype], tokens=fused.shape[0], heads=heads, kv_heads=kv_heads, dim=dim,
                            vdim=vdim, rot_dims=rot_dims, eps=eps, input=fused.data_ptr(), ld=fused.stride(0),
                            q_gamma=_ptr(q_gamma), k_gamma=_ptr(k_gamma), inv_freq=_ptr(inv_freq),
                            q_out=q_out.data_ptr(), ld_q=q_out.stride(0), tok_seq=tok_seq.data_ptr(),
-                           tok_pos=tok_pos.data_ptr(), kv=kv_view))
+                           tok_pos=tok_pos.data_ptr(), kv=kv_view, pairing=1 if neighbours else 0,
+                           norm_span=1 if whole_norm else 0))
 
 
 # --- routed feed-forward ----------------------------------------------------------------------
 
-def route(h, router, correction, top, groups, keep, weights, gate_weight=None, gate=None):
+def route(h, router, correction, top, groups, keep, weights, gate_weight=None, gate=None, score="softmax",
+          group_rank=1, normalize=True):
     """Per row of ``h``: softmax of the float32 router's logits over all experts, the ``top`` experts
     with the largest score + ``correction`` among the best ``keep`` of ``groups`` equal groups (groups
     <= 1: among all), and into ``weights`` [rows, experts] the chosen experts' scores divided by their
-    sum, zero elsewhere.  With ``gate_weight`` [width]: ``gate`` [rows] = sigmoid(gate_weight . h)."""
+    sum, zero elsewhere.  With ``gate_weight`` [width]: ``gate`` [rows] = sigmoid(gate_weight . h).
+    ``score`` "sigmoid": each logit's sigmoid instead of the softmax; ``group_rank`` n: a group's score is the
+    sum of its n best; ``normalize`` False: the chosen experts' scores as they are."""
     _launch(_module("experts"), "bt_route_call",
             RouteCall(dtype=DTYPE_CODES[h.dtype], tokens=h.shape[0], width=router.shape[1], experts=router.shape[0],
                       top=top, groups=groups, keep=keep, h=h.data_ptr(), ldh=h.stride(0), W=router.data_ptr(),
-                      correction=_ptr(correction), gate_w=_ptr(gate_weight), weights=weights.data_ptr(), gate=_ptr(gate)))
+                      correction=_ptr(correction), gate_w=_ptr(gate_weight), weights=weights.data_ptr(), gate=_ptr(gate),
+                      score={"softmax": 0, "sigmoid": 1}[score], group_rank=group_rank, normalize=1 if normalize else 0))
 
 
-def gated_experts(gu, weights, gate, experts, ff, shared_ff, identity, hidden, h=None, identity_out=None):
+def gated_experts(gu, weights, gate, experts, ff, shared_ff, identity, hidden, h=None, identity_out=None, limit=None,
+                  alpha=1.0):
     """hidden[t, e * ff + i] = weights[t, e] * silu(gate_e,i) * up_e,i from the rows ``gu`` of a fused
     gate/up projection (per expert its gate rows, then its up rows; behind the experts the one every
     token uses, weighted by ``gate[t]``); columns behind them are set to zero.  ``identity_out`` (float32
-    [rows, width]) receives (the sum of the identity experts' weights) * h."""
+    [rows, width]) receives (the sum of the identity experts' weights) * h.  With ``limit`` the unit is
+    g' * sigmoid(alpha * g') * (u' + 1), g' = min(gate, limit), u' = clamp(up, -limit, limit), instead of silu(gate) * up."""
     _launch(_module("experts"), "bt_gated_experts_call",
             GatedExpertsCall(dtype=DTYPE_CODES[gu.dtype], tokens=gu.shape[0], experts=experts, ff=ff, shared_ff=shared_ff,
                              identity=identity, hidden_cols=hidden.shape[1], width=h.shape[1] if h is not None else 0,
-                             gu=gu.data_ptr(), ld_gu=gu.stride(0), weights=weights.data_ptr(), gate=_ptr(gate),
+                             gu=gu.data_ptr(), ld_gu=gu.stride(0), weights=_ptr(weights), gate=_ptr(gate),
+                             act=0 if limit is None else 1, limit=limit or 0.0, alpha=alpha,
                              hidden=hidden.data_ptr(), ld_hidden=hidden.stride(0), h=_ptr(h),
                              ldh=h.stride(0) if h is not None else 0, identity_out=_ptr(identity_out)))
+
+
+# --- norms in parts, capped logits -------------------------------------------------------------
+
+def group_norm_output(x, gamma, groups, eps, delta, bias=None, scale=1.0, delta2=None, bias2=None, scale2=1.0, gate=None,
+                      mult=1.0, accumulate=True, cast=None):
+    """x[t] (+)= mult * N(v), v = scale * (sum(delta[:, t]) + bias) + scale2 * (sum(delta2[:, t]) + bias2), times
+    sigmoid(gate[t]) where ``gate`` (float32 logits [tokens, width]) is given; N divides each of ``groups`` equal
+    consecutive parts of the row by its own root mean square and multiplies the whole by ``gamma``.  ``cast``
+    receives the new x in the products' type (zeros behind it)."""
+    def shape(d):
+        if d is None:
+            return 0, 0, 0
+        return (d.shape[0], d.stride(0), d.stride(1)) if d.dim() == 3 else (1, 0, d.stride(0))
+    n1, stride1, ld1 = shape(delta)
+    n2, stride2, ld2 = shape(delta2)
+    tokens, width = x.shape
+    _launch(_module("sublayer"), "bt_group_norm_call",
+            GroupNormCall(cast_dtype=DTYPE_CODES[cast.dtype] if cast is not None else FLOAT32, tokens=tokens, width=width,
+                          groups=groups, n_delta=n1, n_delta2=n2, accumulate=1 if accumulate else 0,
+                          cast_cols=cast.shape[1] if cast is not None else 0, eps=eps, mult=mult, scale=scale, scale2=scale2,
+                          x=x.data_ptr(), delta=_ptr(delta), delta_stride=stride1, ldd=ld1, bias=_ptr(bias),
+                          delta2=_ptr(delta2), delta2_stride=stride2, ldd2=ld2, bias2=_ptr(bias2), gate=_ptr(gate),
+                          ld_gate=gate.stride(0) if gate is not None else 0, gamma=gamma.data_ptr(), cast=_ptr(cast),
+                          ld_cast=cast.stride(0) if cast is not None else 0, rows=None))
+
+
+def group_norm_rows(x, gamma, groups, eps, out, rows=None):
+    """out[r] = N(x[rows[r]]) (every row of x in order without ``rows``), N as in ``group_norm_output``; x stays."""
+    count = rows.numel() if rows is not None else x.shape[0]
+    _launch(_module("sublayer"), "bt_group_norm_call",
+            GroupNormCall(cast_dtype=DTYPE_CODES[out.dtype], tokens=count, width=x.shape[1], groups=groups, n_delta=0,
+                          n_delta2=0, accumulate=0, cast_cols=out.shape[1], eps=eps, mult=1.0, scale=1.0, scale2=1.0,
+                          x=x.data_ptr(), gamma=gamma.data_ptr(), cast=out.data_ptr(), ld_cast=out.stride(0),
+                          rows=_ptr(rows)))
+
+
+def soft_cap(logits, cap):
+    """logits <- cap * tanh(logits / cap), in place (float32 rows)."""
+    _launch(_module("sublayer"), "bt_soft_cap_call",
+            SoftCapCall(rows=logits.shape[0], columns=logits.shape[1], cap=cap, logits=logits.data_ptr(), ld=logits.stride(0)))
+
+
+# --- linear attention with a matrix state -------------------------------------------------------
+
+def keyed_scan(q, k, v, g, out, state, step, heads, kv_heads, dim, vdim, form, beta=None, A_log=None, g_bias=None,
+               lower=None, unit=False, unit_eps=1e-6, q_scale=1.0):
+    """Per head S <- diag(decay) S; S <- S + key u^T; out = S^T query, token after token (csrc/linear_attention.hip).
+    ``form`` "delta": u = sigmoid(beta) (v - S^T key), decay = exp(-exp(A_log) g) from step sizes ``g``, ``q`` and
+    ``k`` rows of ``kv_heads`` heads (made unit vectors per head with ``unit``, q times ``q_scale``).  ``form``
+    "forget": f = lower + (1 - lower) sigmoid(g + g_bias), decay = f, key = 1 - f, query = silu(q), u = v.
+    ``state`` [slots, >= heads * dim * vdim rounded up to 4] float32 is read and left updated."""
+    _launch(_module("linear_attention"), "bt_keyed_scan_call",
+            KeyedScanCall(tokens=v.shape[0], n_seqs=step.n_seqs, heads=heads, kv_heads=kv_heads, dim=dim, vdim=vdim,
+                          form={"delta": 0, "forget": 1}[form], unit=1 if unit else 0, unit_eps=unit_eps, q_scale=q_scale,
+                          q=q.data_ptr(), ld_q=q.stride(0), k=_ptr(k), ld_k=k.stride(0) if k is not None else 0,
+                          v=v.data_ptr(), ld_v=v.stride(0), g=g.data_ptr(), ld_g=g.stride(0), beta=_ptr(beta),
+                          ld_beta=beta.stride(0) if beta is not None else 0, A_log=_ptr(A_log), g_bias=_ptr(g_bias),
+                          lower=_ptr(lower), out=out.data_ptr(), ld_out=out.stride(0), S=state.data_ptr(),
+                          state_stride=state.stride(0), seq_off=step.seq_off.data_ptr(), slots=step.slots.data_ptr()))
+
+
+def head_norm_gate(y, weight, heads, vdim, eps, out, gate=None, mult=1.0):
+    """out[t, h * vdim + i] = mult * y / sqrt(mean_i(y^2) + eps) * weight[i] * sigmoid(gate) per head (no last factor
+    without ``gate``, float32 logits [tokens, heads * vdim]); zeros behind the heads."""
+    _launch(_module("linear_attention"), "bt_head_norm_gate_call",
+            HeadNormGateCall(out_dtype=DTYPE_CODES[out.dtype], tokens=y.shape[0], heads=heads, vdim=vdim,
+                             out_cols=out.shape[1], eps=eps, mult=mult, y=y.data_ptr(), ld_y=y.stride(0), gate=_ptr(gate),
+                             ld_gate=gate.stride(0) if gate is not None else 0, weight=weight.data_ptr(),
+                             out=out.data_ptr(), ld_out=out.stride(0)))

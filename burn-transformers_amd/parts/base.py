@@ -7,6 +7,7 @@
   Embedding    embed(step) -> ResidualStream             (token table and position encoding)
   Readout      logits(h, step) -> float32 [rows, vocab]
   Transform    forward(stream, step)                     (replaces the stream's rows: a projection between runs of layers)
+  Gate         logits(h, step) -> float32 [tokens, width] (a sublayer's output is multiplied by their sigmoid)
   Block        forward(stream, step, memory)             (the arrangement of the parts above)
 
 No part knows which model it is in: it gets its sizes and constants as parameters and its
@@ -31,9 +32,18 @@ from ..kernels import library as K
 @dataclass
 class Delta:
     """A contribution to the residual stream that has not been added yet:
-    sum(partials, dim 0) + bias.  partials: float32 [splits, tokens, width]."""
+    scale * (sum(partials, dim 0) + bias) (+ ``other``, a second term of the same kind, for a sublayer made
+    of two parts side by side).  partials: float32 [splits, tokens, width].  A factor other than one and a
+    second term are understood by norms of a sublayer's output that say so (``takes_weighted_output``);
+    nothing else adds them to the stream."""
     partials: torch.Tensor
     bias: Optional[torch.Tensor] = None
+    scale: float = 1.0
+    other: Optional["Delta"] = None
+
+    @property
+    def plain(self):
+        return self.scale == 1.0 and self.other is None
 
 
 class ResidualStream:
@@ -79,6 +89,9 @@ class ResidualStream:
         return self.x
 
     def add(self, delta):
+        if not delta.plain:
+            raise ValueError("a weighted sum of two parts' outputs joins the stream through a norm of the sublayer's "
+                             "output that takes one (rms_norm's add_output), not as it is")
         if self.pending is not None or self.pending_output is not None:
             self.flush()
         self.pending = delta
@@ -132,8 +145,9 @@ class SublayerOutput(ResidualStream):
     (a ``Delta``), never added to anything, and the block hands it to the norm.  Parts written for the
     residual stream (``stream.add_product``, ``stream.add``, or a returned ``Delta``) run unchanged."""
 
-    def __init__(self):
+    def __init__(self, key="sublayer.partials"):
         super().__init__(None)
+        self.key = key              # the step's buffer for the partial sums (two sublayers side by side: one each)
 
     def add(self, delta):
         if self.pending is not None:
@@ -142,7 +156,7 @@ class SublayerOutput(ResidualStream):
 
     def add_product(self, step, a, weight, bias=None, packed=None):
         splits = stream_product_splits(step, a, weight)
-        partials = step.partial_sums("sublayer.partials", splits, a.shape[0], weight.shape[0])
+        partials = step.partial_sums(self.key, splits, a.shape[0], weight.shape[0])
         K.gemm(a, weight, K.epilogue_f32(partials), splits=splits, packed=packed)
         self.add(Delta(partials, bias))
 
@@ -254,6 +268,15 @@ class Readout(Part):
     takes_deferred_norm = False
 
     def logits(self, h, step):
+        raise NotImplementedError
+
+
+class Gate(Part):
+    """A gate on a sublayer's output, computed from what the sublayer reads: the block hands the logits to
+    the norm of the output, which multiplies by their sigmoid on the way."""
+
+    def logits(self, h, step, key):
+        """float32 [tokens, width]; ``key`` names the step's buffer to use."""
         raise NotImplementedError
 
 

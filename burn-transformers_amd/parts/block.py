@@ -6,7 +6,8 @@ returns it as a Delta, which stays pending until the next norm reads the stream.
 
 output_norm: y = x + m * norm(mixer(x)); z = y + m * norm(feed_forward(y)), the feed-forward
 optional.  The parts read the stream itself; what is normalised is what they add.  ``m`` is the
-block's parameter ``mult``.
+block's parameter ``mult``.  With gates (``mixer_gate``, ``ff_gate``: parts of role "gate") a sublayer's
+output is multiplied, element by element, by sigmoid(gate(x)) before it is normalised: a gated residual.
 
 sandwich_norm: y = x + post(mixer(pre(x))); z = y + post'(feed_forward(pre'(y))), the feed-forward
 optional: a norm before AND behind every sublayer, four norms a layer with tensors of their own.
@@ -78,8 +79,9 @@ class OutputNormBlock(Block):
     """Sublayers that read the residual stream as it is and whose outputs are normalised (and scaled
     by ``mult``) before they join it.  The norms are of a kind with ``add_output`` (rms_norm).  A
     layer without a feed-forward leaves ``ff`` and ``ff_norm`` out."""
-    ROLES = {"mixer": "mixer", "mixer_norm": "norm", "ff": "feed_forward", "ff_norm": "norm"}
-    OPTIONAL = ("ff", "ff_norm")
+    ROLES = {"mixer": "mixer", "mixer_norm": "norm", "ff": "feed_forward", "ff_norm": "norm",
+             "mixer_gate": "gate", "ff_gate": "gate"}
+    OPTIONAL = ("ff", "ff_norm", "mixer_gate", "ff_gate")
     only_launches_kernels = True
 
     def __init__(self, parts, params=None):
@@ -87,6 +89,11 @@ class OutputNormBlock(Block):
         self.mult = float(self.params.get("mult", 1.0))
         if ("ff" in parts) != ("ff_norm" in parts):
             raise ValueError("output_norm block: a feed-forward and its norm come together")
+        if "ff_gate" in parts and "ff" not in parts:
+            raise ValueError("output_norm block: a gate on a feed-forward that is not there")
+        for gate, norm in (("mixer_gate", "mixer_norm"), ("ff_gate", "ff_norm")):
+            if gate in parts and not getattr(parts[norm], "takes_weighted_output", False):
+                raise ValueError(f"output_norm block: {type(parts[norm]).__name__} takes no gate on what it normalises")
         for name in ("mixer_norm", "ff_norm"):
             if name in parts and not hasattr(parts[name], "add_output"):
                 raise ValueError(f"output_norm block: {type(parts[name]).__name__} cannot normalise a sublayer's output")
@@ -94,11 +101,15 @@ class OutputNormBlock(Block):
     def forward(self, stream, step, memory):
         parts = self.parts
         output = SublayerOutput()
-        delta = parts["mixer"].forward(stream.operand(step), step, memory, output)
-        parts["mixer_norm"].add_output(stream, step, delta if delta is not None else output.take(), self.mult)
+        h = stream.operand(step)
+        gate = {"gate": parts["mixer_gate"].logits(h, step, "block.gate")} if "mixer_gate" in parts else {}
+        delta = parts["mixer"].forward(h, step, memory, output)
+        parts["mixer_norm"].add_output(stream, step, delta if delta is not None else output.take(), self.mult, **gate)
         if "ff" in parts:
-            delta = parts["ff"].forward(stream.operand(step), step, output)
-            parts["ff_norm"].add_output(stream, step, delta if delta is not None else output.take(), self.mult)
+            h = stream.operand(step)
+            gate = {"gate": parts["ff_gate"].logits(h, step, "block.gate")} if "ff_gate" in parts else {}
+            delta = parts["ff"].forward(h, step, output)
+            parts["ff_norm"].add_output(stream, step, delta if delta is not None else output.take(), self.mult, **gate)
 
 
 @register("block", "sandwich_norm")

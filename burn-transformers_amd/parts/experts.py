@@ -5,7 +5,11 @@ Parameters: width, experts (experts with tensors), ff (an expert's inner width),
 without tensors whose output is their input; they are the LAST router outputs), top (experts a
 token uses), groups / keep (the experts, identity experts included, form ``groups`` equal groups of
 neighbours, and only experts of the ``keep`` groups with the best score can be chosen; groups <= 1:
-all can), shared_ff (inner width of the expert every token uses; 0: none).
+all can), shared_ff (inner width of the expert every token uses; 0: none), score ("softmax", the default,
+or "sigmoid": each router logit's own sigmoid), group_rank (a group's score is the sum of its so many best
+scores; default 1, its best), normalize (default true; false: the weights are the chosen experts' scores as
+they are), limit and alpha (with a limit an expert's unit is g' * sigmoid(alpha g') * (u' + 1) with
+g' = min(gate h, limit), u' = clamp(up h, -limit, limit), instead of silu(gate h) * (up h)).
 Tensors: router [experts + identity, width] and correction [experts + identity] in float32, per
 expert gate / up [ff, width] and down [width, ff] (``gate_<e>``, ``up_<e>``, ``down_<e>``), and for the
 shared expert shared_gate / shared_up / shared_down and shared_mix [1, width].
@@ -47,6 +51,14 @@ class RoutedExperts(FeedForward):
         self.identity, self.top = int(p.get("identity") or 0), p["top"]
         self.groups, self.keep = int(p.get("groups") or 1), int(p.get("keep") or 1)
         self.shared_ff = int(p.get("shared_ff") or 0)
+        self.score, self.group_rank = p.get("score", "softmax"), int(p.get("group_rank") or 1)
+        self.normalize = bool(p.get("normalize", True))
+        self.limit = float(p["limit"]) if p.get("limit") is not None else None
+        self.alpha = float(p.get("alpha", 1.0))
+        if self.score not in ("softmax", "sigmoid"):
+            raise ValueError(f"routed experts: unknown score {self.score!r}")
+        if self.limit is not None and not self.limit > 0.0:
+            raise ValueError(f"routed experts: the limit {self.limit} must be positive")
         self.outputs = self.experts + self.identity
         if not (0 < self.top <= self.outputs):
             raise ValueError(f"routed experts: {self.top} of {self.outputs} experts a token")
@@ -83,7 +95,8 @@ class RoutedExperts(FeedForward):
         self.inner = self.experts * self.ff + self.shared_ff
         self.hidden_cols = operand_columns(self.inner, dtype)
         self.fused_cols = operand_columns(2 * self.inner, dtype)      # (rows of the fused product's output start where 16-byte stores may)
-        self.in_weight = pad_rows(torch.cat(rows), self.fused_cols)                           # [2 * inner (+ zero rows), width]
+        # [2 * inner (+ zero rows), width (+ zero columns, where the rows it multiplies carry them)]
+        self.in_weight = pad_columns(pad_rows(torch.cat(rows), self.fused_cols), operand_columns(self.width, dtype))
         self.down_weight = pad_columns(torch.cat(columns, dim=1), self.hidden_cols)           # [width, inner (+ zeros)]
         on_gpu = self.in_weight.is_cuda
         self.in_packed = K.PackedWeight(self.in_weight) if on_gpu else None
@@ -96,7 +109,8 @@ class RoutedExperts(FeedForward):
         tokens = h.shape[0]
         weights = step.buffer("experts.weights", tokens, self.outputs, "float32")
         mix = step.buffer("experts.mix", tokens, 1, "float32") if self.shared_ff else None
-        K.route(h, self.router, self.correction, self.top, self.groups, self.keep, weights, self.shared_mix, mix)
+        K.route(h, self.router, self.correction, self.top, self.groups, self.keep, weights, self.shared_mix, mix,
+                score=self.score, group_rank=self.group_rank, normalize=self.normalize)
         fused = step.buffer("experts.fused", tokens, self.fused_cols, step.dtype)
         K.gemm(h, self.in_weight, K.epilogue_store(fused), packed=self.in_packed)
         hidden = step.buffer("experts.hidden", tokens, self.hidden_cols, step.dtype)
@@ -104,6 +118,7 @@ class RoutedExperts(FeedForward):
         extra = 1 if self.identity else 0
         partials = step.partial_sums("experts.partials", splits + extra, tokens, self.width)
         K.gated_experts(fused, weights, mix, self.experts, self.ff, self.shared_ff, self.identity, hidden,
-                        h=h if self.identity else None, identity_out=partials[splits] if self.identity else None)
+                        h=h if self.identity else None, identity_out=partials[splits] if self.identity else None,
+                        limit=self.limit, alpha=self.alpha)
         K.gemm(hidden, self.down_weight, K.epilogue_f32(partials[:splits]), splits=splits, packed=self.down_packed)
         return Delta(partials, None)

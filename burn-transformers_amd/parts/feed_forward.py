@@ -10,6 +10,10 @@ element by element and N(v) = v / sqrt(mean(v^2) + eps) over a token's whole inn
 numbers are the tensor ``act_coefficients``, ``eps`` a parameter.  It needs a whole row, so the up
 projection leaves 32-bit sums and a kernel of its own applies it.
 
+gated_dense: down(silu(gate x) * (up x)), no biases.  Parameters width, inner; tensors gate_weight and
+up_weight [inner, width], down_weight [width, inner].  ONE product with the two matrices laid one behind the
+other, the kernel of the routed experts' units for the single unit every token uses, and the down product.
+
 The MFMA kernels read operands 16 bytes at a time, so an inner width that is no multiple of 8 is
 padded once, when the part is built: zero rows (and zero bias) in the up projection give
 act(0) = 0 in the padded columns, which meet zero columns of the down projection.
@@ -18,7 +22,7 @@ act(0) = 0 in the padded columns, which meet zero columns of the down projection
 import torch
 
 from ..kernels import library as K
-from .base import FeedForward, packed_for_stream
+from .base import FeedForward, operand_columns, packed_for_stream, pad_columns, pad_rows
 from .registry import register
 
 
@@ -71,3 +75,37 @@ class DenseFeedForward(FeedForward):
             hidden = step.buffer("feed_forward.hidden", tokens, self.padded, step.dtype)
         K.gemm(h, self.up_weight, K.epilogue_act(hidden, self.activation, self.up_bias), packed=self.up_packed)
         stream.add_product(step, hidden, self.down_weight, self.down_bias, packed=self.down_packed)
+
+
+@register("feed_forward", "gated_dense")
+class GatedDenseFeedForward(FeedForward):
+    takes_deferred_norm = False
+    only_launches_kernels = True
+
+    def __init__(self, params, tensors):
+        super().__init__(params, tensors)
+        self.width, self.inner = params["width"], params["inner"]
+        gate, up, down = tensors["gate_weight"], tensors["up_weight"], tensors["down_weight"]
+        if tuple(gate.shape) != (self.inner, self.width) or tuple(up.shape) != (self.inner, self.width) or \
+                tuple(down.shape) != (self.width, self.inner):
+            raise ValueError(f"gated feed-forward: projections {tuple(gate.shape)}, {tuple(up.shape)}, {tuple(down.shape)} do "
+                             f"not fit width {self.width} and inner width {self.inner}")
+        dtype = gate.dtype
+        columns = operand_columns(self.width, dtype)
+        self.hidden_cols = operand_columns(self.inner, dtype)
+        self.fused_cols = operand_columns(2 * self.inner, dtype)
+        self.in_weight = pad_columns(pad_rows(torch.cat([gate, up]), self.fused_cols), columns)
+        self.down_weight = pad_columns(down, self.hidden_cols)
+        self.in_packed = K.PackedWeight(self.in_weight) if self.in_weight.is_cuda else None
+        self.down_packed = packed_for_stream(self.down_weight) if self.down_weight.is_cuda else None
+
+    def kernel_modules(self, dtype):
+        return ("experts",)
+
+    def forward(self, h, step, stream):
+        tokens = h.shape[0]
+        fused = step.buffer("feed_forward.fused", tokens, self.fused_cols, step.dtype)
+        K.gemm(h, self.in_weight, K.epilogue_store(fused), packed=self.in_packed)
+        hidden = step.buffer("feed_forward.hidden", tokens, self.hidden_cols, step.dtype)
+        K.gated_experts(fused, None, None, 0, 1, self.inner, 0, hidden)
+        stream.add_product(step, hidden, self.down_weight, packed=self.down_packed)

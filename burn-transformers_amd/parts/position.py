@@ -3,7 +3,9 @@
 learned_positions: x0[t] = tokens[id[t]] + positions[pos[t]]  (src/models/gpt2/model.rs:447-448);
 the table's length bounds a sequence's length.  token_only: x0[t] = scale * tokens[id[t]] (for models
 whose position encoding lives in the mixer; ``scale`` defaults to 1; with ``keep_origin`` the rows
-are also kept beside the stream, ``stream.origin``, for parts that read the embedding's output again).  normalized_tokens: x0[t] = rms_norm(tokens[id[t]]) with
+are also kept beside the stream, ``stream.origin``, for parts that read the embedding's output again; with
+``keep_operand`` a bfloat16 model also gets the rows in the products' type, ``stream.cast``, for layers whose
+sublayers multiply by the stream itself).  normalized_tokens: x0[t] = rms_norm(tokens[id[t]]) with
 a scale of its own (stored as its distance from ``offset``), for models that normalise the
 embedding before the first layer; it also leaves the stream's copy in the products' type.
 """
@@ -41,6 +43,8 @@ class TokenEmbedding(Embedding):
         self.width, self.vocab_size = params["width"], params["vocab_size"]
         self.max_positions = params.get("max_positions", 2 ** 31 - 1)
         self.scale, self.keep_origin = float(params.get("scale", 1.0)), bool(params.get("keep_origin", False))
+        # for layers whose sublayers multiply by the stream itself: its rows in the products' type beside it
+        self.keep_operand = bool(params.get("keep_operand", False))
         self.token_table = tensors["tokens"]
         if tuple(self.token_table.shape) != (self.vocab_size, self.width):
             raise ValueError("embedding: the table does not have the configured sizes")
@@ -48,9 +52,12 @@ class TokenEmbedding(Embedding):
     def embed(self, step):
         x = step.buffer("stream.x", step.n_tokens, self.width, "float32")
         origin = step.buffer("stream.origin", step.n_tokens, self.width, "float32") if self.keep_origin else None
-        K.embed(step.tok_ids, None, self.token_table, None, x, scale=self.scale, copy=origin)
+        cast = None
+        if self.keep_operand and step.dtype != x.dtype:
+            cast = step.buffer("stream.operand", step.n_tokens, operand_columns(self.width, step.dtype), step.dtype)
+        K.embed(step.tok_ids, None, self.token_table, None, x, scale=self.scale, copy=origin, cast=cast)
         stream = ResidualStream(x)
-        stream.origin = origin
+        stream.origin, stream.cast = origin, cast
         return stream
 
 

@@ -1,5 +1,6 @@
 """Readout: logits = h . table^T in float32, no bias; the table is [vocab, width] and may be
-the token table itself (src/models/gpt2/model.rs:500-513, src/operations.rs:675-728)."""
+the token table itself (src/models/gpt2/model.rs:500-513, src/operations.rs:675-728).  Parameter
+``soft_cap`` (default none): logits <- cap * tanh(logits / cap), in 32-bit."""
 
 from ..kernels import library as K
 from .base import Readout
@@ -15,6 +16,9 @@ class LinearReadout(Readout):
         super().__init__(params, tensors)
         self.width, self.vocab_size = params["width"], params["vocab_size"]
         self.weight = tensors["weight"]
+        self.soft_cap = float(params.get("soft_cap") or 0.0)
+        if self.soft_cap < 0.0 or self.soft_cap != self.soft_cap:
+            raise ValueError(f"readout: the logits' cap {self.soft_cap} must be positive")
         if tuple(self.weight.shape) != (self.vocab_size, self.width):
             raise ValueError(f"readout: table is {tuple(self.weight.shape)}, expected "
                              f"{(self.vocab_size, self.width)}")
@@ -25,4 +29,6 @@ class LinearReadout(Readout):
     def logits(self, h, step):
         out = step.buffer("readout.logits", h.shape[0], self.vocab_size, "float32")
         K.gemm(h, self.weight, K.epilogue_f32(out), packed=self.packed)
+        if self.soft_cap:
+            K.soft_cap(out, self.soft_cap)
         return out

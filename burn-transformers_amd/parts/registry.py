@@ -4,9 +4,9 @@ Adding a part means writing a class with the interface of ``parts/base.py`` and 
 under a new kind; plans may then name it layer by layer.
 """
 
-MIXERS, FEED_FORWARDS, NORMS, EMBEDDINGS, READOUTS, BLOCKS, TRANSFORMS = {}, {}, {}, {}, {}, {}, {}
+MIXERS, FEED_FORWARDS, NORMS, EMBEDDINGS, READOUTS, BLOCKS, TRANSFORMS, GATES = {}, {}, {}, {}, {}, {}, {}, {}
 _TABLES = {"mixer": MIXERS, "feed_forward": FEED_FORWARDS, "norm": NORMS, "embedding": EMBEDDINGS,
-           "readout": READOUTS, "block": BLOCKS, "transform": TRANSFORMS}
+           "readout": READOUTS, "block": BLOCKS, "transform": TRANSFORMS, "gate": GATES}
 
 
 def register(role, kind, cls=None, replace=False):

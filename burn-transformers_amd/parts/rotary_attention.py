@@ -9,8 +9,12 @@ query and key head are turned, channel i with channel i + rot_dims / 2, by the a
 f_i), rot_base (f_i = rot_base^(-2 i / rot_dims)), rot_scaling (None, or factor / low / high /
 original: frequencies whose wavelength is beyond original / low are divided by factor, those whose
 wavelength is below original / high are kept, and between the two the division is blended in
-linearly in original / wavelength), window and chunk (which earlier keys a query sees, as in
-``parts/attention.py``).  Tensors: q_weight [heads * dim, width], k_weight [kv_heads * dim, width],
+linearly in original / wavelength), rot_pairing ("halves", the default: channel i with channel i + rot_dims / 2;
+"neighbours": channel 2 i with channel 2 i + 1), norm_span ("head", the default; "whole": the root mean square
+is taken over a token's whole query (key) projection before it is split into heads, and the scales ``q_norm`` /
+``k_norm`` are [heads * dim] / [kv_heads * dim]), window and chunk (which earlier keys a query sees, as in
+``parts/attention.py``).  Optional tensor ``sink`` [heads]: a learned logit per head that stands in the softmax's
+denominator beside the keys', with no key and no value.  Tensors: q_weight [heads * dim, width], k_weight [kv_heads * dim, width],
 v_weight [kv_heads * vdim, width], out_weight [width, heads * vdim], no biases.
 
 One step: ONE product with the three projections laid one behind the other leaves 32-bit sums; a
@@ -27,7 +31,7 @@ import torch
 
 from ..kernels import library as K
 from .attention import CausalSelfAttention
-from .base import Mixer, packed_for_stream
+from .base import Mixer, operand_columns, packed_for_stream, pad_columns
 from .registry import register
 
 
@@ -63,12 +67,18 @@ class RotaryAttention(CausalSelfAttention):
             raise ValueError(f"rotary attention: {self.rot_dims} turned channels must be even and at most the head size {self.dim}")
         shapes = {"q_weight": (self.heads * self.dim, self.width), "k_weight": (self.kv_heads * self.dim, self.width),
                   "v_weight": (self.kv_heads * self.vdim, self.width), "out_weight": (self.width, self.heads * self.vdim)}
+        self.neighbours = {"halves": False, "neighbours": True}[p.get("rot_pairing", "halves")]
+        self.whole_norm = {"head": False, "whole": True}[p.get("norm_span", "head")]
         if p.get("head_norm", True):
-            shapes.update(q_norm=(self.dim,), k_norm=(self.dim,))
+            shapes.update(q_norm=(self.heads * self.dim,), k_norm=(self.kv_heads * self.dim,)) if self.whole_norm else \
+                shapes.update(q_norm=(self.dim,), k_norm=(self.dim,))
+        if "sink" in tensors:
+            shapes["sink"] = (self.heads,)
         for role, shape in shapes.items():
             if tuple(tensors[role].shape) != shape:
                 raise ValueError(f"rotary attention: {role} is {tuple(tensors[role].shape)}, expected {shape}")
         self.q_norm, self.k_norm = tensors.get("q_norm"), tensors.get("k_norm")
+        self.sink = tensors["sink"].float().contiguous() if "sink" in tensors else None
         dtype = tensors["q_weight"].dtype
         bf16 = dtype == torch.bfloat16
         # the cached head: the larger of the two head sizes, in the steps of 16 the MFMA kernels take
@@ -80,7 +90,8 @@ class RotaryAttention(CausalSelfAttention):
         self.plain_decode = bf16 and self.heads // self.kv_heads > 16
         self.n_q, self.n_kv = self.heads * self.head_dim, self.kv_heads * self.head_dim
         self.fused_cols = (self.heads + self.kv_heads) * self.dim + self.kv_heads * self.vdim
-        self.qkv_weight = torch.cat([tensors["q_weight"], tensors["k_weight"], tensors["v_weight"]]).contiguous()
+        self.qkv_weight = pad_columns(torch.cat([tensors["q_weight"], tensors["k_weight"], tensors["v_weight"]]),
+                                      operand_columns(self.width, dtype))
         # the output projection reads heads of head_dim: its columns are spread, zeros between them
         out = tensors["out_weight"]
         spread = out.new_zeros(self.width, self.heads, self.head_dim)
@@ -106,7 +117,8 @@ class RotaryAttention(CausalSelfAttention):
         K.gemm(h, self.qkv_weight, K.epilogue_f32(fused), packed=self.qkv_packed)
         q = step.buffer("attention.q", tokens, self.n_q, step.dtype)
         K.head_rotary(fused, self.heads, self.kv_heads, self.dim, self.vdim, self.rot_dims, self.inv_freq,
-                      self.q_norm, self.k_norm, self.eps, q, step.tok_seq, step.tok_pos, kv, step.dtype)
+                      self.q_norm, self.k_norm, self.eps, q, step.tok_seq, step.tok_pos, kv, step.dtype,
+                      neighbours=self.neighbours, whole_norm=self.whole_norm)
         plain = self.plain_only or (self.plain_decode and step.decode)
         if step.decode and step.dtype_is_bf16 and K.Chunked.wanted(tokens) and not plain:
             mixed = K.Chunked.take(step, "attention.mixed", tokens, self.n_q, step.dtype)
@@ -117,7 +129,7 @@ class RotaryAttention(CausalSelfAttention):
             partial = step.buffer("attention.partial", step.n_seqs * self.heads * runs, self.head_dim + 2, "float32")
         args = K.attention_args(q, mixed, kv, step.tok_seq, step.tok_pos, step.seq_off, step.seq_start,
                                 self.heads, step.n_seqs, step.max_count, self.scale, self.window, partial,
-                                chunk=self.chunk)
+                                chunk=self.chunk, sink=self.sink)
         # (the bfloat16 decode kernel takes up to 16 query heads on a cached head; beyond, the plain kernel)
         K.attention(args, step.dtype, step.decode, impl="plain" if plain else "auto")
         stream.add_product(step, mixed, self.out_weight, None, packed=self.out_packed)

@@ -25,8 +25,11 @@ LAYOUTS = ("in_out", "out_in", "table", "vector", "int")
 
 @dataclass(frozen=True)
 class TensorSpec:
+    """``shape``: an extent is a number, or a string that names a size which only the checkpoint gives (the rank
+    of a low-rank projection, say): any positive extent fits, and every tensor that names the same string must
+    agree on it."""
     name: str
-    shape: Tuple[int, ...]
+    shape: Tuple[object, ...]
     layout: str
 
     def __post_init__(self):
@@ -66,6 +69,19 @@ class WeightError(ValueError):
         super().__init__("\n".join(lines))
 
 
+def fits(stored, wanted, free):
+    """Whether a stored shape fits a spec's; ``free`` collects what the named extents turned out to be."""
+    if len(stored) != len(wanted):
+        return False
+    for have, want in zip(stored, wanted):
+        if isinstance(want, str):
+            if have < 1 or free.setdefault(want, have) != have:
+                return False
+        elif have != want:
+            return False
+    return True
+
+
 def detect_prefix(names, contract, where):
     """The one namespace that holds the anchor tensor (src/models/gpt2/checkpoint.rs:61-71)."""
     if contract.anchor is None:
@@ -89,11 +105,11 @@ def check(entries, contract, where, listed_only=()):
     ignored = [re.compile(pattern) for pattern in contract.ignored]
     wanted = {prefix + spec.name: spec for spec in contract.tensors}
     missing = [name for name in wanted if name not in names]
-    unexpected, mismatched, stored_aliases = [], [], []
+    unexpected, mismatched, stored_aliases, free = [], [], [], {}
     for name in sorted(names):
         if name in wanted:
             spec, entry = wanted[name], entries[name]
-            if tuple(entry.shape) != tuple(spec.shape):
+            if not fits(tuple(entry.shape), tuple(spec.shape), free):
                 mismatched.append(f"{name}: stored {entry.dtype}{list(entry.shape)}, the model needs {list(spec.shape)}")
             elif spec.layout == "int" and entry.dtype in FLOAT_DTYPES:
                 mismatched.append(f"{name}: an integer table is stored as {entry.dtype}")
