@@ -214,3 +214,13 @@ def forward(ids, weights, config, streams=None):
     logits = group_norm(x, w["final.norm"], groups, eps) @ w["head"].T
     cap = config.get("logit_softcap")
     return cap * torch.tanh(logits / cap) if cap else logits
+
+
+def greedy(ids, weights, config, new_tokens):
+    """The `new_tokens` tokens with the largest logit, each fed back."""
+    ids, made = list(ids), []
+    for _ in range(new_tokens):
+        token = int(forward(ids, weights, config)[-1].argmax())
+        made.append(token)
+        ids.append(token)
+    return made
