@@ -1,7 +1,7 @@
 """Throughput of GPT-2 generation on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers 48] [--dtype bf16]
-                    [--repetitions 10] [--workload xl|small|medium|sweep|salopel|kodatar] [--model xl|medium|small]
+                    [--repetitions 10] [--workload xl|small|medium|sweep|salopel|kodatar|rotutar] [--model xl|medium|small]
                     [--kernel-batches 1,64] [--sweep-part all|decode|prompts] [--no-points] [--no-kernels] [--no-own]
 
 The default workload (``xl``) has the layer sizes of GPT-2 XL with random weights: a batch of 8
@@ -49,6 +49,9 @@ a real model's, beside GPT-2 at equal width, depth, feed-forward and vocabulary:
 throughput and each model's classes of kernels, one JSON line per width.
 ``--workload kodatar`` does the same for the third family, Kodatar (rotary attention in chunks, routed
 experts, a stretch of layers that runs twice), beside GPT-2 at equal width, runs of layers and vocabulary.
+``--workload rotutar`` runs the fourth family, Rotutar (linear attention with a matrix state, window attention
+with a sink beside a delta rule, gated sublayer outputs, routed experts), beside Salopel, the library's closest
+family, at equal width, layers and vocabulary.
 """
 
 import argparse
@@ -235,6 +238,20 @@ def _class_of(name, call):
         return f"gated_experts {call.tokens}x{call.hidden_cols}", call.tokens * call.hidden_cols * 3 * element, 0.0
     if short == "join_rows":
         return f"join_rows {call.tokens}x{call.width}", call.tokens * call.width * (8 + 2 * (4 if call.out_dtype == 0 else 2)), 0.0
+    if short == "keyed_scan":           # state read and written; queries, keys, decays, values in, read-outs out
+        state = call.n_seqs * call.heads * call.dim * call.vdim * 8
+        rows = call.tokens * ((2 * call.kv_heads if call.form == 0 else call.heads) * call.dim + call.heads * (call.dim + 2 * call.vdim)) * 4
+        return f"keyed_scan {call.tokens}x{call.heads}x{call.dim}x{call.vdim}", state + rows, \
+            (7.0 if call.form == 0 else 5.0) * call.tokens * call.heads * call.dim * call.vdim
+    if short == "head_norm_gate":
+        return f"head_norm_gate {call.tokens}x{call.heads * call.vdim}", \
+            call.tokens * call.heads * call.vdim * ((8 if call.gate else 4) + (4 if call.out_dtype == 0 else 2)), 0.0
+    if short == "group_norm":
+        terms = call.n_delta + call.n_delta2 + (1 if call.gate else 0)
+        return f"group_norm {call.tokens}x{call.width}", (terms + 2) * call.tokens * call.width * 4 + \
+            (call.tokens * call.cast_cols * 2 if call.cast else 0), 0.0
+    if short == "soft_cap":
+        return f"soft_cap {call.rows}x{call.columns}", call.rows * call.columns * 8, 0.0
     if short == "gated_norm":
         return f"gated_norm {call.tokens}x{call.channels}", call.tokens * call.channels * 10, 0.0
     return short, 0, 0.0
@@ -570,6 +587,35 @@ def kodatar_config(width, layers, vocab):
             "layers": [dict(layer) for _ in range(layers - third)]}
 
 
+def rotutar_config(width, layers, vocab):
+    """Rotutar at layer sizes that resemble a real model's: groups of four layers (a forget-gate layer with a
+    dense feed-forward of 4 x width, one with experts, the pair of window attention and delta rule with experts, a
+    forget-gate layer with experts); heads of 128 everywhere, the attention's on a quarter as many key/value heads
+    with a window of 512, the delta rule's queries and keys on half as many heads, four taps, low ranks of 64;
+    eight experts of the model's width in four groups of which two stay open, a token uses two."""
+    heads = max(4, width // 128)
+    forget = {"heads": heads, "dim": 128, "vdim": 128}
+    pair = {"left": {"heads": heads, "kv_heads": heads // 4, "dim": 128, "vdim": 128, "scale": 128 ** -0.5,
+                     "rot": {"dims": 128, "base": 10000.0}, "mask": {"size": 512}},
+            "right": {"heads": heads, "kv_heads": heads // 2, "dim": 128, "vdim": 128, "conv": 4, "rank": 64},
+            "left_scale": 1.0, "right_scale": 1.0}
+    experts = {"kind": "moe", "expert": {"ff": width, "limit": 7.0},
+               "router": {"experts": 8, "top": 2, "groups": {"count": 4, "keep": 2}}}
+    group = [{"type": "hgrn2", "mixer": forget, "mlp": {"kind": "dense", "ff": 4 * width}},
+             {"type": "hgrn2", "mixer": forget, "mlp": experts}, {"type": "parallel", "mixer": pair, "mlp": experts},
+             {"type": "hgrn2", "mixer": forget, "mlp": experts}]
+    return {"architecture": "Rotutar", "vocab": vocab, "width": width, "logit_softcap": 30.0, "norm": {"eps": 1e-5, "groups": 2},
+            "layers": [dict(group[i % 4]) for i in range(layers)]}
+
+
+def run_rotutar(args):
+    """Rotutar beside the library's closest family, Salopel (recurrent layers with a state per sequence, norms of
+    the sublayers' outputs), at equal width, layers and vocabulary."""
+    heads = lambda width: max(4, width // 128)
+    run_beside_gpt2(args, "rotutar", rotutar_config, lambda width: (2 * 128 * (heads(width) // 4), 128 * heads(width)),
+                    other=("salopel", salopel_config, lambda width: (2 * 128, 128 * min(16, width // 64))))
+
+
 def run_salopel(args):
     """Prompt and decode throughput of Salopel beside GPT-2 at equal width, depth, feed-forward and
     vocabulary, with each model's classes of kernels on their own.  One JSON line per width."""
@@ -582,9 +628,10 @@ def run_kodatar(args):
                     lambda width: (2 * 128 * (max(4, width // 128) // 4), 128 * max(4, width // 128)))
 
 
-def run_beside_gpt2(args, family, config_of, attention_sizes):
+def run_beside_gpt2(args, family, config_of, attention_sizes, other=None):
     """``attention_sizes(width)``: (cached values a token and layer, columns of a token's queries), for
-    the attention kernels' bytes and flops."""
+    the attention kernels' bytes and flops.  ``other``: (family, its configuration, its attention sizes) of the
+    model that runs beside, GPT-2 without."""
     import torch
 
     import burn_transformers_amd as bt
@@ -592,13 +639,14 @@ def run_beside_gpt2(args, family, config_of, attention_sizes):
     layers, batch, prompt_len, steps = args.layers or 12, args.batch, 512, min(args.steps, 64)
     vocab = 32000
     for width in (1024, 2048):
-        cached, columns = attention_sizes(width)
-        line = {"workload": f"{family} beside gpt2", "width": width, "layers": layers, "dtype": dtype, "batch": batch,
+        beside = other[0] if other else "gpt2"
+        line = {"workload": f"{family} beside {beside}", "width": width, "layers": layers, "dtype": dtype, "batch": batch,
                 "prompt_len": prompt_len, "decode_steps": steps, "data": "synthetic token ids, random weights"}
-        for name in (family, "gpt2"):
-            if name == family:
-                config = config_of(width, layers, vocab)
+        for name in (family, beside):
+            if name == family or other:
+                config = (config_of if name == family else other[1])(width, layers, vocab)
                 model = build_salopel(config, dtype)
+                cached, columns = (attention_sizes if name == family else other[2])(width)
             else:
                 config = dict(XL, n_layer=layers, n_embd=width, n_head=width // 64, n_inner=4 * width, vocab_size=vocab,
                               n_positions=2048)
@@ -616,15 +664,17 @@ def run_beside_gpt2(args, family, config_of, attention_sizes):
                 prompts = synthetic_prompts(batch, context - 1, vocab, seed=7)
                 slots = [engine.open() for _ in prompts]
                 engine.step(list(zip(slots, prompts)))
-                kv = batch * context * cached * ELEMENT_BYTES[dtype] if name == family else batch * context * 2 * width * ELEMENT_BYTES[dtype]
-                flops = 4.0 * batch * context * (columns if name == family else width)
+                if name == "gpt2":
+                    cached, columns = 2 * width, width
+                kv = batch * context * cached * ELEMENT_BYTES[dtype]
+                flops = 4.0 * batch * context * columns
                 result["decode_kernels"] = kernel_classes(engine, [(slot, [5]) for slot in slots], kv, flops, PEAK_FLOPS[dtype])
                 for slot in slots:
                     engine.close(slot)
                 prompts = synthetic_prompts(PREFILL_SEQS, PREFILL_LEN, vocab, seed=8)
                 slots = [engine.open() for _ in prompts]
                 tokens = PREFILL_SEQS * PREFILL_LEN
-                per_token = columns if name == family else width
+                per_token = columns
                 result["prefill_kernels"] = kernel_classes(engine, list(zip(slots, prompts)), 4 * tokens * per_token * ELEMENT_BYTES[dtype],
                                                            PREFILL_SEQS * 2.0 * per_token * PREFILL_LEN * (PREFILL_LEN + 1),
                                                            PEAK_FLOPS[dtype], replays=10)
@@ -648,7 +698,7 @@ def main():
     parser.add_argument("--kernel-batches", default="", help="further batch sizes whose decode kernel classes are timed, e.g. 1,64")
     parser.add_argument("--dtype", choices=["bf16", "fp32"], default=None)
     parser.add_argument("--repetitions", type=int, default=10, help="measured repetitions, each on fresh sequences")
-    parser.add_argument("--workload", choices=["xl", "small", "medium", "sweep", "salopel", "kodatar"], default="xl")
+    parser.add_argument("--workload", choices=["xl", "small", "medium", "sweep", "salopel", "kodatar", "rotutar"], default="xl")
     parser.add_argument("--sweep-part", choices=["all", "decode", "prompts"], default="all",
                         help="which table of --workload sweep to run")
     parser.add_argument("--no-points", action="store_true", help="skip batch 1 and 64")
@@ -661,8 +711,8 @@ def main():
     if args.repetitions < 1:
         parser.error("--repetitions must be at least 1")
     args.kernel_batches = [int(b) for b in args.kernel_batches.split(",") if b]
-    if args.workload in ("salopel", "kodatar"):
-        (run_salopel if args.workload == "salopel" else run_kodatar)(args)
+    if args.workload in ("salopel", "kodatar", "rotutar"):
+        {"salopel": run_salopel, "kodatar": run_kodatar, "rotutar": run_rotutar}[args.workload](args)
         return
     if args.layers is None:
         args.layers = XL["n_layer"] if args.workload == "sweep" else MODELS[args.model]["n_layer"]

@@ -51,12 +51,26 @@ struct KeyedScanCall {
 // One wave per (4 value channels of a head, sequence): sixteen lanes share a channel, lane j of them owns
 // the key channels j, j + 16, ... of its column of S in registers.  A work-group is four waves with four
 // channels each of the same head: they share the run of (g, k, q) in LDS.
+// A run is up to 2048 / NP tokens (NP = 16 R key channels, padded), so that a thread stages KS_LOADS entries
+// of it: every load of a run is issued before the first is used (a loop of single loads is waited for once
+// per trip), and the NEXT run's loads are issued before this run's tokens are walked, so memory's latency
+// hides behind the recurrence.
 #define KS_WAVES 4
+#define KS_THREADS (64 * KS_WAVES)
+#define KS_LOADS 8
+
+template <int R>
+struct KsRun {
+  static constexpr int NP = 16 * R;
+  static constexpr int MOST = 2048 / NP > 64 ? 64 : 2048 / NP;     // tokens of a run
+  static constexpr int TOK_LOADS = (MOST * 4 + 63) / 64;           // (v, beta) pairs a lane stages
+};
 
 template <int R, int FORM>
-__global__ void __launch_bounds__(64 * KS_WAVES) keyed_scan_kernel(KeyedScanCall c, int chunk, int tiles) {
+__global__ void __launch_bounds__(KS_THREADS) keyed_scan_kernel(KeyedScanCall c, int chunk, int tiles) {
   extern __shared__ __attribute__((aligned(16))) float lds[];
-  constexpr int NP = 16 * R;
+  constexpr int NP = KsRun<R>::NP, TOK_LOADS = KsRun<R>::TOK_LOADS;
+  constexpr int ROWS_A_TURN = KS_THREADS / NP;                                // tokens that the threads' entries of one turn span
   float4* gkq = reinterpret_cast<float4*>(lds);                               // [chunk][NP]: decay, key, query
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, sub = lane & 15, pl = lane >> 4;
   float2* tok = reinterpret_cast<float2*>(lds + (size_t)chunk * NP * 4) + (size_t)wave * chunk * 4;   // [waves][chunk][4]: v, beta
@@ -75,38 +89,69 @@ __global__ void __launch_bounds__(64 * KS_WAVES) keyed_scan_kernel(KeyedScanCall
   }
   const float rate = FORM == 0 ? -expf(c.A_log[head]) : 0.f;
   float* ocol = c.out + head * c.vdim + (live ? p : 0);
+  // a thread's entries of a run are key channel `n` of the tokens row0, row0 + ROWS_A_TURN, ...
+  const int n = threadIdx.x % NP, row0 = threadIdx.x / NP;
+  const bool in_head = n < c.dim;
+  const int nc = in_head ? n : 0;
+  const int col_g = head * c.dim + nc, col_k = shared * c.dim + nc;
+  float low = 0.f, bias = 0.f;
+  if (FORM == 1) {
+    low = c.lower[col_g];
+    bias = c.g_bias ? c.g_bias[col_g] : 0.f;
+  }
+  const int ch = tile * 4 + (lane & 3);                   // the value channel of a lane's (v, beta) pairs
+  const int chc = ch < c.vdim ? ch : 0;
+  float rg[KS_LOADS], rk[KS_LOADS], rq[KS_LOADS], rv[TOK_LOADS], rb[TOK_LOADS];
+  // issues the loads of the run that starts at token t0 (rows beyond the run read its last token and are dropped)
+  auto fetch = [&](int t0, int count) {
+#pragma unroll
+    for (int j = 0; j < KS_LOADS; ++j) {
+      const int i = min(row0 + j * ROWS_A_TURN, count - 1);
+      const int64_t t = t0 + i;
+      rg[j] = c.g[t * c.ld_g + col_g];
+      rq[j] = c.q[t * c.ld_q + (FORM == 0 ? col_k : col_g)];
+      rk[j] = FORM == 0 ? c.k[t * c.ld_k + col_k] : 0.f;
+    }
+#pragma unroll
+    for (int j = 0; j < TOK_LOADS; ++j) {
+      const int i = min((lane >> 2) + 16 * j, count - 1);
+      const int64_t t = t0 + i;
+      rv[j] = c.v[t * c.ld_v + head * c.vdim + chc];
+      rb[j] = FORM == 0 ? c.beta[t * c.ld_beta + head] : 0.f;
+    }
+  };
+  if (first < last) fetch(first, min(chunk, last - first));
   for (int t0 = first; t0 < last; t0 += chunk) {
     const int count = min(chunk, last - t0);
-    __syncthreads();
-    for (int e = threadIdx.x; e < count * NP; e += 64 * KS_WAVES) {
-      const int i = e / NP, n = e % NP;
-      float4 in = make_float4(0.f, 0.f, 0.f, 0.f);
-      if (n < c.dim) {
-        const int64_t t = t0 + i;
-        if (FORM == 0) {
-          in.x = expf(rate * c.g[t * c.ld_g + head * c.dim + n]);
-          in.y = c.k[t * c.ld_k + shared * c.dim + n];
-          in.z = c.q[t * c.ld_q + shared * c.dim + n];
-        } else {
-          const int col = head * c.dim + n;
-          const float low = c.lower[col];
-          const float raw = c.g[t * c.ld_g + col] + (c.g_bias ? c.g_bias[col] : 0.f);
-          const float f = low + (1.0f - low) / (1.0f + expf(-raw));
-          in.x = f;
-          in.y = 1.0f - f;
-          in.z = silu_f(c.q[t * c.ld_q + col]);
+    __syncthreads();                                       // the run before has been walked
+#pragma unroll
+    for (int j = 0; j < KS_LOADS; ++j) {
+      const int i = row0 + j * ROWS_A_TURN;
+      if (i < count) {
+        float4 in = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (in_head) {
+          if (FORM == 0) {
+            in.x = expf(rate * rg[j]);
+            in.y = rk[j];
+            in.z = rq[j];
+          } else {
+            const float f = low + (1.0f - low) / (1.0f + expf(-(rg[j] + bias)));
+            in.x = f;
+            in.y = 1.0f - f;
+            in.z = silu_f(rq[j]);
+          }
         }
+        gkq[i * NP + n] = in;
       }
-      gkq[e] = in;
     }
-    for (int e = lane; e < count * 4; e += 64) {
-      const int i = e >> 2, ch = tile * 4 + (e & 3);
-      const int64_t t = t0 + i;
-      const float v = ch < c.vdim ? c.v[t * c.ld_v + head * c.vdim + ch] : 0.f;
-      const float b = FORM == 0 ? 1.0f / (1.0f + expf(-c.beta[t * c.ld_beta + head])) : 1.0f;
-      tok[e] = make_float2(v, b);
+#pragma unroll
+    for (int j = 0; j < TOK_LOADS; ++j) {
+      const int i = (lane >> 2) + 16 * j;
+      if (i < count)
+        tok[i * 4 + (lane & 3)] = make_float2(ch < c.vdim ? rv[j] : 0.f, FORM == 0 ? 1.0f / (1.0f + expf(-rb[j])) : 1.0f);
     }
     __syncthreads();
+    if (t0 + chunk < last) fetch(t0 + chunk, min(chunk, last - t0 - chunk));      // in flight while this run is walked
     if (FORM == 0 && c.unit) {          // q and k as unit vectors: sixteen lanes take a token
       for (int i = threadIdx.x >> 4; i < count; i += 4 * KS_WAVES) {
         float sk = 0.f, sq = 0.f;
@@ -116,52 +161,65 @@ __global__ void __launch_bounds__(64 * KS_WAVES) keyed_scan_kernel(KeyedScanCall
           sk = fmaf(e.y, e.y, sk);
           sq = fmaf(e.z, e.z, sq);
         }
-        const float rk = 1.0f / sqrtf(sum_of_16_lanes(sk) + c.unit_eps);
-        const float rq = c.q_scale / sqrtf(sum_of_16_lanes(sq) + c.unit_eps);
+        const float rk_ = 1.0f / sqrtf(sum_of_16_lanes(sk) + c.unit_eps);
+        const float rq_ = c.q_scale / sqrtf(sum_of_16_lanes(sq) + c.unit_eps);
 #pragma unroll
         for (int r = 0; r < R; ++r) {
           float4 e = gkq[i * NP + sub + 16 * r];
-          e.y *= rk;
-          e.z *= rq;
+          e.y *= rk_;
+          e.z *= rq_;
           gkq[i * NP + sub + 16 * r] = e;
         }
       }
       __syncthreads();
     }
     if (!works) continue;
-    for (int i = 0; i < count; ++i) {
-      const float2 vb = tok[i * 4 + pl];
-      float4 in[R];
+    // a token's inputs are read from LDS while the token before it is worked on: a wave is alone on its SIMD,
+    // so nothing else hides that latency
+    float4 in[R];
+    float2 vb = tok[pl];
 #pragma unroll
-      for (int r = 0; r < R; ++r) in[r] = gkq[i * NP + sub + 16 * r];
+    for (int r = 0; r < R; ++r) in[r] = gkq[sub + 16 * r];
+#pragma unroll 4
+    for (int i = 0; i < count; ++i) {
+      const int ahead = min(i + 1, count - 1);
+      float4 next[R];
+      const float2 vb_next = tok[ahead * 4 + pl];
+#pragma unroll
+      for (int r = 0; r < R; ++r) next[r] = gkq[ahead * NP + sub + 16 * r];
       float u = vb.x;
       if (FORM == 0) {
-        float answered = 0.f;
+        float answered = 0.f, answered_odd = 0.f;          // (two sums: half as long a chain of dependent adds)
 #pragma unroll
         for (int r = 0; r < R; ++r) {
           S[r] *= in[r].x;
-          answered = fmaf(S[r], in[r].y, answered);
+          if (r & 1) answered_odd = fmaf(S[r], in[r].y, answered_odd);
+          else answered = fmaf(S[r], in[r].y, answered);
         }
-        u = vb.y * (vb.x - sum_of_16_lanes(answered));
+        u = vb.y * (vb.x - sum_of_16_lanes(answered + answered_odd));
       } else {
 #pragma unroll
         for (int r = 0; r < R; ++r) S[r] *= in[r].x;
       }
-      float acc = 0.f;
+      float acc = 0.f, acc_odd = 0.f;
 #pragma unroll
       for (int r = 0; r < R; ++r) {
         S[r] = fmaf(in[r].y, u, S[r]);
-        acc = fmaf(S[r], in[r].z, acc);
+        if (r & 1) acc_odd = fmaf(S[r], in[r].z, acc_odd);
+        else acc = fmaf(S[r], in[r].z, acc);
       }
-      const float o = sum_of_16_lanes(acc);
+      const float o = sum_of_16_lanes(acc + acc_odd);
       if (live && sub == 0) ocol[(int64_t)(t0 + i) * c.ld_out] = o;
+      vb = vb_next;
+#pragma unroll
+      for (int r = 0; r < R; ++r) in[r] = next[r];
     }
   }
   if (!works) return;
 #pragma unroll
   for (int r = 0; r < R; ++r) {
-    const int n = sub + 16 * r;
-    if (n < c.dim) held[(int64_t)n * 4] = S[r];
+    const int nn = sub + 16 * r;
+    if (nn < c.dim) held[(int64_t)nn * 4] = S[r];
   }
 }
 
@@ -169,8 +227,8 @@ template <int R>
 static void launch_keyed_scan(hipStream_t stream, const KeyedScanCall& c) {
   const int per_token = 4 * 16 * R + 8 * KS_WAVES;
   const int tiles = (c.vdim + 3) / 4, groups = (tiles + KS_WAVES - 1) / KS_WAVES;
-  const int chunk = scan_chunk(per_token, c.tokens);
-  dim3 grid(groups, c.heads, c.n_seqs), block(64 * KS_WAVES);
+  const int chunk = c.tokens < KsRun<R>::MOST ? c.tokens : KsRun<R>::MOST;
+  dim3 grid(groups, c.heads, c.n_seqs), block(KS_THREADS);
   const size_t lds = (size_t)chunk * per_token * sizeof(float);
   if (c.form == 0)
     hipLaunchKernelGGL((keyed_scan_kernel<R, 0>), grid, block, lds, stream, c, chunk, tiles);

@@ -443,6 +443,126 @@ __global__ void __launch_bounds__(256) group_norm_kernel(GroupNormCall c) {
       cast[(int64_t)t * c.ld_cast + col] = from_float<T>(0.f);
 }
 
+// The same for rows of up to 256 * KMAX columns: a thread's columns live in registers, and every load of a
+// thread (partial sums of both terms, biases, the gate, the stream, the scale) is issued before the first is
+// used and none stands behind a branch of its own, so a row costs one round trip to memory (a decode step has
+// few rows: one row's latency is its time).  The parts' sums of squares meet in LDS, a wave a part.
+template <typename T, int KMAX>
+__global__ void __launch_bounds__(256) group_norm_small_kernel(GroupNormCall c) {
+  extern __shared__ float row_buf[];          // [width], then [groups] reciprocal roots
+  float* rstd = row_buf + c.width;
+  const int t = blockIdx.x;
+  const bool from_stream = c.n_delta == 0;
+  const int source = from_stream && c.rows ? c.rows[t] : t;
+  float* xr = c.x + (int64_t)source * c.width;
+  float v[KMAX], w[KMAX], xv[KMAX], g[KMAX], gt[KMAX];
+  int cc[KMAX];
+#pragma unroll
+  for (int k = 0; k < KMAX; ++k) {
+    const int col = threadIdx.x + 256 * k;
+    cc[k] = col < c.width ? col : 0;
+  }
+  const float* bias = c.bias ? c.bias : c.gamma;           // (read in any case, used only where there is one)
+  const float* bias2 = c.bias2 ? c.bias2 : c.gamma;
+  const float* gate = c.gate ? c.gate + (int64_t)t * c.ld_gate : c.gamma;
+#pragma unroll
+  for (int k = 0; k < KMAX; ++k) {
+    g[k] = c.gamma[cc[k]];
+    xv[k] = xr[cc[k]];
+    v[k] = bias[cc[k]];
+    w[k] = bias2[cc[k]];
+    gt[k] = gate[cc[k]];
+  }
+#pragma unroll
+  for (int k = 0; k < KMAX; ++k) {
+    v[k] = c.bias ? v[k] : 0.f;
+    w[k] = c.bias2 ? w[k] : 0.f;
+  }
+  if (from_stream) {
+#pragma unroll
+    for (int k = 0; k < KMAX; ++k) v[k] = xv[k];
+  } else {
+    const float* row = c.delta + (int64_t)t * c.ldd;
+    for (int s0 = 0; s0 < c.n_delta; s0 += 4) {            // four partial sums at a time, all their loads together
+      float part[4][KMAX];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int sc = s0 + u < c.n_delta ? s0 + u : c.n_delta - 1;
+#pragma unroll
+        for (int k = 0; k < KMAX; ++k) part[u][k] = row[sc * c.delta_stride + cc[k]];
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+#pragma unroll
+        for (int k = 0; k < KMAX; ++k) v[k] += s0 + u < c.n_delta ? part[u][k] : 0.f;
+    }
+    const float* row2 = c.delta2 + (int64_t)t * c.ldd2;
+    for (int s0 = 0; s0 < c.n_delta2; s0 += 4) {
+      float part[4][KMAX];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int sc = s0 + u < c.n_delta2 ? s0 + u : c.n_delta2 - 1;
+#pragma unroll
+        for (int k = 0; k < KMAX; ++k) part[u][k] = row2[sc * c.delta2_stride + cc[k]];
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+#pragma unroll
+        for (int k = 0; k < KMAX; ++k) w[k] += s0 + u < c.n_delta2 ? part[u][k] : 0.f;
+    }
+#pragma unroll
+    for (int k = 0; k < KMAX; ++k) {
+      v[k] *= c.scale;
+      if (c.n_delta2 > 0) v[k] = fmaf(c.scale2, w[k], v[k]);
+      if (c.gate) v[k] *= 1.0f / (1.0f + expf(-gt[k]));
+    }
+  }
+#pragma unroll
+  for (int k = 0; k < KMAX; ++k) {
+    const int col = threadIdx.x + 256 * k;
+    if (col < c.width) row_buf[col] = v[k];
+  }
+  __syncthreads();
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = blockDim.x >> 6;
+  const int per = c.width / c.groups;
+  for (int part = wave; part < c.groups; part += waves) {
+    float squares = 0.f;
+    for (int i = lane; i < per; i += 64) squares = fmaf(row_buf[part * per + i], row_buf[part * per + i], squares);
+    squares = wave_sum(squares);
+    if (lane == 0) rstd[part] = 1.0f / sqrtf(squares / (float)per + c.eps);
+  }
+  __syncthreads();
+  T* cast = static_cast<T*>(c.cast);
+#pragma unroll
+  for (int k = 0; k < KMAX; ++k) {
+    const int col = threadIdx.x + 256 * k;
+    if (col < c.width) {
+      float y = v[k] * rstd[col / per] * g[k];
+      if (!from_stream) {
+        y *= c.mult;
+        if (c.accumulate) y += xv[k];
+        xr[col] = y;
+      }
+      if (cast) cast[(int64_t)t * c.ld_cast + col] = from_float<T>(y);
+    }
+  }
+  if (cast)
+    for (int col = c.width + threadIdx.x; col < c.cast_cols; col += blockDim.x)
+      cast[(int64_t)t * c.ld_cast + col] = from_float<T>(0.f);
+}
+
+template <typename T>
+static void launch_group_norm(hipStream_t stream, const GroupNormCall& c) {
+  const size_t lds = (size_t)(c.width + c.groups) * sizeof(float);
+  dim3 grid(c.tokens), block(256);
+  if (c.width <= 1024)
+    hipLaunchKernelGGL((group_norm_small_kernel<T, 4>), grid, block, lds, stream, c);
+  else if (c.width <= 2048)
+    hipLaunchKernelGGL((group_norm_small_kernel<T, 8>), grid, block, lds, stream, c);
+  else
+    hipLaunchKernelGGL(group_norm_kernel<T>, grid, block, lds, stream, c);
+}
+
 BT_EXPORT int bt_group_norm_call(void* stream, const GroupNormCall* c) {
   if (c->tokens <= 0) return BT_OK;
   if (c->width <= 0 || c->width > 15360) BT_REFUSE("group_norm: width %d outside 1..15360", c->width);
@@ -457,12 +577,10 @@ BT_EXPORT int bt_group_norm_call(void* stream, const GroupNormCall* c) {
     BT_REFUSE("group_norm: a copy of %d columns in rows of %lld does not hold width %d", c->cast_cols,
               (long long)c->ld_cast, c->width);
   if (c->gate && c->ld_gate < c->width) BT_REFUSE("group_norm: the gate's rows are shorter than the width");
-  const size_t lds = (size_t)(c->width + c->groups) * sizeof(float);
-  dim3 grid(c->tokens), block(256);
   if (c->cast_dtype == 0)
-    hipLaunchKernelGGL(group_norm_kernel<float>, grid, block, lds, (hipStream_t)stream, *c);
+    launch_group_norm<float>((hipStream_t)stream, *c);
   else
-    hipLaunchKernelGGL(group_norm_kernel<bf16_t>, grid, block, lds, (hipStream_t)stream, *c);
+    launch_group_norm<bf16_t>((hipStream_t)stream, *c);
   return bt_check_launch("group_norm");
 }
 
