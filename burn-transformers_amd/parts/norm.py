@@ -49,9 +49,11 @@ class _KernelNorm(Norm):
 
     def apply(self, stream, step, rows=None, chunked=False):
         count = rows.numel() if rows is not None else stream.x.shape[0]
-        if self.groups > 1:
+        if self.groups > 1 or (self.KIND == "rms_norm" and operand_columns(self.width, step.dtype) != self.width):
+            # (also rows that a product reads 16 bytes at a time and that are no multiple of that long: zeros behind them)
             stream.flush()
-            out = step.buffer("norm.out" if rows is None else "norm.selected", count, self.width, step.dtype)
+            out = step.buffer("norm.out" if rows is None else "norm.selected", count, operand_columns(self.width, step.dtype),
+                              step.dtype)
             K.group_norm_rows(stream.x, self.weight, self.groups, self.eps, out, rows=rows)
             return out
         if chunked and K.Chunked.wanted(count) and self.width % 4 == 0:
@@ -75,7 +77,7 @@ class _KernelNorm(Norm):
         return out
 
     def deferred_possible(self, step, rows):
-        return self.groups == 1 and step.dtype_is_bf16 and K.Normalized.worth_it(rows, self.width)
+        return self.groups == 1 and step.dtype_is_bf16 and self.width % 8 == 0 and K.Normalized.worth_it(rows, self.width)
 
     def deferred(self, stream, step):
         if stream.pending is not None or stream.pending_output is not None or \

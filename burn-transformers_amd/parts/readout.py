@@ -3,7 +3,7 @@ the token table itself (src/models/gpt2/model.rs:500-513, src/operations.rs:675-
 ``soft_cap`` (default none): logits <- cap * tanh(logits / cap), in 32-bit."""
 
 from ..kernels import library as K
-from .base import Readout
+from .base import Readout, operand_columns, pad_columns
 from .registry import register
 
 
@@ -24,11 +24,14 @@ class LinearReadout(Readout):
                              f"{(self.vocab_size, self.width)}")
         # a second copy for steps of few rows, which read the table and little else (the token
         # embedding looks rows up in the table as it is stored)
-        self.packed = K.PackedWeight(self.weight) if self.weight.is_cuda else None
+        # (rows that a bfloat16 product reads 16 bytes at a time: a width that is no multiple of that gets zero columns,
+        # which meet the zero columns behind the normalised rows)
+        self.matrix = pad_columns(self.weight, operand_columns(self.width, self.weight.dtype))
+        self.packed = K.PackedWeight(self.matrix) if self.weight.is_cuda else None
 
     def logits(self, h, step):
         out = step.buffer("readout.logits", h.shape[0], self.vocab_size, "float32")
-        K.gemm(h, self.weight, K.epilogue_f32(out), packed=self.packed)
+        K.gemm(h, self.matrix, K.epilogue_f32(out), packed=self.packed)
         if self.soft_cap:
             K.soft_cap(out, self.soft_cap)
         return out

@@ -75,7 +75,11 @@ MANY_HEADS = model_config([layer(side_by_side(window_attention(20, 1, 16, 16, 0.
                                               delta(2, 1, 16, 16, 2, rank=4), 1.0, 1.0), dense(24))], width=48, vocab=71, groups=2)
 WIDE_HEADS = model_config([layer(side_by_side(window_attention(2, 1, 144, 20, 0.08, rot_dims=100, window=30),
                                               delta(1, 1, 200, 70, 3, rank=4), 1.0, 1.0))], width=32, vocab=53, groups=1)
-CONFIGS = {"basic": (BASIC, 1), "odd": (ODD, 2), "forget": (FORGET_ONLY, 3), "attention": (ATTENTION_ONLY, 4),
+# nothing a multiple of eight: a width of 36 in three parts, heads of 10, 12, 6 and 20, feed-forwards of 10 and 22
+UNALIGNED = model_config([layer(forget(2, 10, 6), moe(3, 10, 2, 1.0)),
+                          layer(side_by_side(window_attention(2, 1, 12, 20, 0.3, rot_dims=6, window=9),
+                                             delta(2, 2, 10, 6, 3, rank=3), 1.0, 1.0), dense(22))], width=36, vocab=53, groups=3)
+CONFIGS = {"unaligned": (UNALIGNED, 11), "basic": (BASIC, 1), "odd": (ODD, 2), "forget": (FORGET_ONLY, 3), "attention": (ATTENTION_ONLY, 4),
            "delta": (DELTA_ONLY, 5), "dense": (DENSE_ONLY, 6), "experts": (EXPERTS_ONLY, 7), "long": (LONG, 8),
            "many_heads": (MANY_HEADS, 9), "wide_heads": (WIDE_HEADS, 10)}
 

@@ -43,7 +43,7 @@ def whole(engine, ids):
                                           ("delta", [1, 2, 3, 4, 5, 70, 200]), ("dense", [1, 17, 80]),
                                           ("experts", [1, 2, 33, 90]), ("basic", [1, 2, 23, 24, 25, 49, 130]),
                                           ("odd", [1, 6, 7, 8, 99, 101, 210]), ("many_heads", [1, 50, 100]),
-                                          ("wide_heads", [1, 31, 90])])
+                                          ("wide_heads", [1, 31, 90]), ("unaligned", [1, 2, 10, 70])])
 def test_each_mechanism_and_each_request_whole(name, dtype, lengths):
     engine = engine_for(name, dtype)
     for ids in prompts_for(name, lengths):
@@ -82,7 +82,7 @@ def test_residual_stream_after_every_layer():
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("name,length,tail", [("basic", 80, 40), ("odd", 110, 20), ("attention", 140, 80), ("delta", 9, 8),
-                                              ("forget", 70, 30), ("many_heads", 100, 30), ("wide_heads", 90, 40)])
+                                              ("forget", 70, 30), ("many_heads", 100, 30), ("wide_heads", 90, 40), ("unaligned", 30, 20)])
 def test_prompt_then_token_by_token(name, dtype, length, tail):
     """The last tokens one by one through the cache and the state give what the whole prompt gives; the tails
     let the window pass over decoded tokens."""
