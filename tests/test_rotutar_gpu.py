@@ -134,8 +134,8 @@ def test_unequal_batch_decoded_together_then_slots_and_blocks_reused(name, dtype
     """Requests of unequal length in one step, decoded together while the shorter ones end; then a
     second batch in the slots, blocks and state rows the first gave back."""
     engine = engine_for(name, dtype, max_tokens=1024)
-    for round_, lengths in enumerate([[1, 70, 33, 129], [64, 5, 90]]):
-        prompts = prompts_for(name, lengths, seed=20 + round_)
+    for batch_, lengths in enumerate([[1, 70, 33, 129], [64, 5, 90]]):
+        prompts = prompts_for(name, lengths, seed=20 + batch_)
         tails = [12, 5, 9, 3][:len(prompts)]
         extra = [prompts_for(name, [t], seed=30 + i)[0] for i, t in enumerate(tails)]
         slots = [engine.open() for _ in prompts]
@@ -154,7 +154,7 @@ def test_unequal_batch_decoded_together_then_slots_and_blocks_reused(name, dtype
                 if t + 1 == tails[i]:
                     engine.close(slots[i])
         for i, p in enumerate(prompts):
-            check(torch.cat(got[i]), plain_logits(name, p + extra[i], dtype=dtype), dtype, f"{name} round {round_} request {i}")
+            check(torch.cat(got[i]), plain_logits(name, p + extra[i], dtype=dtype), dtype, f"{name} batch {batch_} request {i}")
         engine.cache.ledger.check()
     assert not engine.cache.ledger.live_slots()
 
