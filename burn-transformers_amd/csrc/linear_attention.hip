@@ -46,11 +46,19 @@ struct KeyedScanCall {
   int64_t state_stride;
   const int* seq_off;     // [n_seqs + 1]
   const int* slots;       // [n_seqs]
+  // form 1 only: long sequences are cut into spans of at least `span` tokens that are scanned side by side (see
+  // "Spans" in scan.h; the forget gate's step is a diagonal decay and a write, which is linear in S; the delta
+  // rule's is not diagonal and walks its sequences in order).  0: never; max_count is the most tokens a sequence
+  // of the step brings, carry the room for the spans' states: (tokens / span + 2 n_seqs + 1) blocks of a slot's
+  // state and heads * dim products of decays
+  int span;
+  int max_count;
+  float* carry;
 };
 
-// One wave per (4 value channels of a head, sequence): sixteen lanes share a channel, lane j of them owns
-// the key channels j, j + 16, ... of its column of S in registers.  A work-group is four waves with four
-// channels each of the same head: they share the run of (g, k, q) in LDS.
+// One wave per (4 value channels of a head, sequence): sixteen lanes share a channel, each owns R key channels
+// of its column of S in registers.  A work-group is four waves with four channels each of the same head: they
+// share the run of decays, queries and keys in LDS.
 // A run is up to 2048 / NP tokens (NP = 16 R key channels, padded), so that a thread stages KS_LOADS entries
 // of it: every load of a run is issued before the first is used (a loop of single loads is waited for once
 // per trip), and the NEXT run's loads are issued before this run's tokens are walked, so memory's latency
@@ -62,30 +70,75 @@ struct KeyedScanCall {
 template <int R>
 struct KsRun {
   static constexpr int NP = 16 * R;
+  static constexpr int V = R < 4 ? R : 4;                          // floats a lane reads at a time
   static constexpr int MOST = 2048 / NP > 64 ? 64 : 2048 / NP;     // tokens of a run
   static constexpr int TOK_LOADS = (MOST * 4 + 63) / 64;           // (v, beta) pairs a lane stages
 };
 
-template <int R, int FORM>
+// Decays, queries and keys of a run lie in LDS as planes of [tokens][NP] floats (the forget gate's keys are
+// 1 - decay and have no plane: every wave reads a token's whole row of every plane, and with several waves to a
+// SIMD those reads are what bounds a token's time).  Lane j of the sixteen that share a value channel owns the
+// key channels (16 i + j) V + e, i < R / V, e < V: it reads V neighbouring floats at a time, and neighbouring
+// lanes read neighbouring vectors.
+template <int R, int V>
+__device__ __forceinline__ int ks_channel(int sub, int r) { return (16 * (r / V) + sub) * V + r % V; }
+
+template <int R, int V>
+__device__ __forceinline__ void ks_read(const float* row, int sub, float* out) {
+#pragma unroll
+  for (int i = 0; i < R / V; ++i) {
+    const float* at = row + (16 * i + sub) * V;
+    if (V == 4) {
+      const float4 x = *reinterpret_cast<const float4*>(at);
+      out[4 * i] = x.x; out[4 * i + 1] = x.y; out[4 * i + 2] = x.z; out[4 * i + 3] = x.w;
+    } else if (V == 2) {
+      const float2 x = *reinterpret_cast<const float2*>(at);
+      out[2 * i] = x.x; out[2 * i + 1] = x.y;
+    } else {
+      out[i] = at[0];
+    }
+  }
+}
+
+// phase 0: whole sequences, from and to the slot's state.  1: spans from zero, leaving their end states and the
+// products of their decays, no read-outs.  3: spans from the carried states, writing read-outs, leaving no state.
+template <int R, int FORM, int PHASE>
 __global__ void __launch_bounds__(KS_THREADS) keyed_scan_kernel(KeyedScanCall c, int chunk, int tiles) {
+  constexpr int phase = PHASE;
   extern __shared__ __attribute__((aligned(16))) float lds[];
-  constexpr int NP = KsRun<R>::NP, TOK_LOADS = KsRun<R>::TOK_LOADS;
+  constexpr int NP = KsRun<R>::NP, V = KsRun<R>::V, TOK_LOADS = KsRun<R>::TOK_LOADS;
   constexpr int ROWS_A_TURN = KS_THREADS / NP;                                // tokens that the threads' entries of one turn span
-  float4* gkq = reinterpret_cast<float4*>(lds);                               // [chunk][NP]: decay, key, query
+  constexpr int PLANES = FORM == 0 ? 3 : 2;
+  float* G = lds;                                                             // [chunk][NP] decays
+  float* Q = lds + (size_t)chunk * NP;                                        // [chunk][NP] queries
+  float* Kp = lds + (size_t)2 * chunk * NP;                                   // [chunk][NP] keys (delta rule)
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, sub = lane & 15, pl = lane >> 4;
-  float2* tok = reinterpret_cast<float2*>(lds + (size_t)chunk * NP * 4) + (size_t)wave * chunk * 4;   // [waves][chunk][4]: v, beta
-  const int tile = min((int)blockIdx.x * KS_WAVES + wave, tiles - 1), head = blockIdx.y, seq = blockIdx.z;
+  float2* tok = reinterpret_cast<float2*>(lds + (size_t)PLANES * chunk * NP) + (size_t)wave * chunk * 4;   // [waves][chunk][4]: v, beta
+  const int tile = min((int)blockIdx.x * KS_WAVES + wave, tiles - 1), head = blockIdx.y;
+  const int seq = blockIdx.z % c.n_seqs, part = blockIdx.z / c.n_seqs;
   const bool works = (int)blockIdx.x * KS_WAVES + wave < tiles;
   const int p = tile * 4 + pl;
   const bool live = works && p < c.vdim;
   const int shared = FORM == 0 ? head / (c.heads / c.kv_heads) : head;
-  const int first = c.seq_off[seq], last = c.seq_off[seq + 1];
-  float* held = c.S + (int64_t)c.slots[seq] * c.state_stride + ((int64_t)head * tiles + tile) * c.dim * 4 + pl;
-  float S[R];
+  int first = c.seq_off[seq], last = c.seq_off[seq + 1];
+  const int64_t in_slot = ((int64_t)head * tiles + tile) * c.dim * 4 + pl;        // where this lane's column of S starts
+  float* held = c.S + (int64_t)c.slots[seq] * c.state_stride + in_slot;
+  float* products = nullptr;                              // phase 1: where this span's products of decays go
+  if (phase) {
+    first += part * c.span;
+    if (first >= last) return;                            // (the whole work-group: no barrier has been met)
+    last = min(first + c.span, last);
+    const int64_t state_floats = (int64_t)c.heads * tiles * c.dim * 4, per_span = state_floats + (int64_t)c.heads * c.dim;
+    float* mine = c.carry + span_block(c.seq_off, seq, c.span, part) * per_span;
+    held = (phase == 1 ? mine : mine - per_span) + in_slot;
+    products = mine + state_floats + (int64_t)head * c.dim;
+  }
+  float S[R], P[R];
 #pragma unroll
   for (int r = 0; r < R; ++r) {
-    const int n = sub + 16 * r;
-    S[r] = n < c.dim ? held[(int64_t)n * 4] : 0.f;
+    const int n = ks_channel<R, V>(sub, r);
+    S[r] = n < c.dim && phase != 1 ? held[(int64_t)n * 4] : 0.f;
+    P[r] = 1.0f;
   }
   const float rate = FORM == 0 ? -expf(c.A_log[head]) : 0.f;
   float* ocol = c.out + head * c.vdim + (live ? p : 0);
@@ -109,7 +162,7 @@ __global__ void __launch_bounds__(KS_THREADS) keyed_scan_kernel(KeyedScanCall c,
       const int i = min(row0 + j * ROWS_A_TURN, count - 1);
       const int64_t t = t0 + i;
       rg[j] = c.g[t * c.ld_g + col_g];
-      rq[j] = c.q[t * c.ld_q + (FORM == 0 ? col_k : col_g)];
+      rq[j] = PHASE == 1 ? 0.f : c.q[t * c.ld_q + (FORM == 0 ? col_k : col_g)];
       rk[j] = FORM == 0 ? c.k[t * c.ld_k + col_k] : 0.f;
     }
 #pragma unroll
@@ -128,20 +181,19 @@ __global__ void __launch_bounds__(KS_THREADS) keyed_scan_kernel(KeyedScanCall c,
     for (int j = 0; j < KS_LOADS; ++j) {
       const int i = row0 + j * ROWS_A_TURN;
       if (i < count) {
-        float4 in = make_float4(0.f, 0.f, 0.f, 0.f);
+        float decay = 0.f, query = 0.f;
         if (in_head) {
           if (FORM == 0) {
-            in.x = expf(rate * rg[j]);
-            in.y = rk[j];
-            in.z = rq[j];
+            decay = expf(rate * rg[j]);
+            query = rq[j];
           } else {
-            const float f = low + (1.0f - low) / (1.0f + expf(-(rg[j] + bias)));
-            in.x = f;
-            in.y = 1.0f - f;
-            in.z = silu_f(rq[j]);
+            decay = low + (1.0f - low) / (1.0f + expf(-(rg[j] + bias)));
+            query = PHASE == 1 ? 0.f : silu_f(rq[j]);
           }
         }
-        gkq[i * NP + n] = in;
+        G[i * NP + n] = decay;
+        if (PHASE != 1) Q[i * NP + n] = query;
+        if (FORM == 0) Kp[i * NP + n] = in_head ? rk[j] : 0.f;
       }
     }
 #pragma unroll
@@ -154,21 +206,20 @@ __global__ void __launch_bounds__(KS_THREADS) keyed_scan_kernel(KeyedScanCall c,
     if (t0 + chunk < last) fetch(t0 + chunk, min(chunk, last - t0 - chunk));      // in flight while this run is walked
     if (FORM == 0 && c.unit) {          // q and k as unit vectors: sixteen lanes take a token
       for (int i = threadIdx.x >> 4; i < count; i += 4 * KS_WAVES) {
-        float sk = 0.f, sq = 0.f;
+        float kk[R], qq[R], sk = 0.f, sq = 0.f;
+        ks_read<R, V>(Kp + i * NP, sub, kk);
+        ks_read<R, V>(Q + i * NP, sub, qq);
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-          const float4 e = gkq[i * NP + sub + 16 * r];
-          sk = fmaf(e.y, e.y, sk);
-          sq = fmaf(e.z, e.z, sq);
+          sk = fmaf(kk[r], kk[r], sk);
+          sq = fmaf(qq[r], qq[r], sq);
         }
         const float rk_ = 1.0f / sqrtf(sum_of_16_lanes(sk) + c.unit_eps);
         const float rq_ = c.q_scale / sqrtf(sum_of_16_lanes(sq) + c.unit_eps);
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-          float4 e = gkq[i * NP + sub + 16 * r];
-          e.y *= rk_;
-          e.z *= rq_;
-          gkq[i * NP + sub + 16 * r] = e;
+          Kp[i * NP + ks_channel<R, V>(sub, r)] = kk[r] * rk_;
+          Q[i * NP + ks_channel<R, V>(sub, r)] = qq[r] * rq_;
         }
       }
       __syncthreads();
@@ -176,64 +227,116 @@ __global__ void __launch_bounds__(KS_THREADS) keyed_scan_kernel(KeyedScanCall c,
     if (!works) continue;
     // a token's inputs are read from LDS while the token before it is worked on: a wave is alone on its SIMD,
     // so nothing else hides that latency
-    float4 in[R];
+    float g[R], k[R], q[R];
     float2 vb = tok[pl];
-#pragma unroll
-    for (int r = 0; r < R; ++r) in[r] = gkq[sub + 16 * r];
+    ks_read<R, V>(G, sub, g);
+    if (PHASE != 1) ks_read<R, V>(Q, sub, q);
+    if (FORM == 0) ks_read<R, V>(Kp, sub, k);
 #pragma unroll 4
     for (int i = 0; i < count; ++i) {
       const int ahead = min(i + 1, count - 1);
-      float4 next[R];
+      float g_next[R], k_next[R], q_next[R];
       const float2 vb_next = tok[ahead * 4 + pl];
-#pragma unroll
-      for (int r = 0; r < R; ++r) next[r] = gkq[ahead * NP + sub + 16 * r];
+      ks_read<R, V>(G + ahead * NP, sub, g_next);
+      if (PHASE != 1) ks_read<R, V>(Q + ahead * NP, sub, q_next);
+      if (FORM == 0) ks_read<R, V>(Kp + ahead * NP, sub, k_next);
       float u = vb.x;
       if (FORM == 0) {
         float answered = 0.f, answered_odd = 0.f;          // (two sums: half as long a chain of dependent adds)
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-          S[r] *= in[r].x;
-          if (r & 1) answered_odd = fmaf(S[r], in[r].y, answered_odd);
-          else answered = fmaf(S[r], in[r].y, answered);
+          S[r] *= g[r];
+          if (r & 1) answered_odd = fmaf(S[r], k[r], answered_odd);
+          else answered = fmaf(S[r], k[r], answered);
         }
         u = vb.y * (vb.x - sum_of_16_lanes(answered + answered_odd));
       } else {
 #pragma unroll
-        for (int r = 0; r < R; ++r) S[r] *= in[r].x;
+        for (int r = 0; r < R; ++r) {
+          k[r] = 1.0f - g[r];
+          S[r] *= g[r];
+          if (PHASE == 1) P[r] *= g[r];
+        }
       }
-      float acc = 0.f, acc_odd = 0.f;
+      if (PHASE == 1) {                                     // a span from zero leaves its state only: no read-out
 #pragma unroll
-      for (int r = 0; r < R; ++r) {
-        S[r] = fmaf(in[r].y, u, S[r]);
-        if (r & 1) acc_odd = fmaf(S[r], in[r].z, acc_odd);
-        else acc = fmaf(S[r], in[r].z, acc);
+        for (int r = 0; r < R; ++r) S[r] = fmaf(k[r], u, S[r]);
+      } else {
+        float acc = 0.f, acc_odd = 0.f;
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+          S[r] = fmaf(k[r], u, S[r]);
+          if (r & 1) acc_odd = fmaf(S[r], q[r], acc_odd);
+          else acc = fmaf(S[r], q[r], acc);
+        }
+        const float o = sum_of_16_lanes(acc + acc_odd);
+        if (live && sub == 0) ocol[(int64_t)(t0 + i) * c.ld_out] = o;
       }
-      const float o = sum_of_16_lanes(acc + acc_odd);
-      if (live && sub == 0) ocol[(int64_t)(t0 + i) * c.ld_out] = o;
       vb = vb_next;
 #pragma unroll
-      for (int r = 0; r < R; ++r) in[r] = next[r];
+      for (int r = 0; r < R; ++r) {
+        g[r] = g_next[r];
+        if (PHASE != 1) q[r] = q_next[r];
+        if (FORM == 0) k[r] = k_next[r];
+      }
     }
   }
-  if (!works) return;
+  if (!works || phase == 3) return;
 #pragma unroll
   for (int r = 0; r < R; ++r) {
-    const int nn = sub + 16 * r;
+    const int nn = ks_channel<R, V>(sub, r);
     if (nn < c.dim) held[(int64_t)nn * 4] = S[r];
+    if (nn < c.dim && phase == 1 && blockIdx.x == 0 && wave == 0 && pl == 0) products[nn] = P[r];
   }
+}
+
+// C_k = P_k C_(k-1) + E_k along every sequence, in place; C_(-1), the state the sequence came with, is kept in
+// front of its spans, and the last C goes into the slot.
+__global__ void __launch_bounds__(256) keyed_carry_kernel(KeyedScanCall c, int tiles) {
+  const int seq = blockIdx.y;
+  const int64_t index = (int64_t)blockIdx.x * blockDim.x + threadIdx.x, size = (int64_t)c.heads * tiles * c.dim * 4;
+  if (index >= size) return;
+  const int count = c.seq_off[seq + 1] - c.seq_off[seq];
+  const int spans = (count + c.span - 1) / c.span;
+  const int64_t per_span = size + (int64_t)c.heads * c.dim;
+  float* block = c.carry + span_block(c.seq_off, seq, c.span, 0) * per_span;
+  float* slot = c.S + (int64_t)c.slots[seq] * c.state_stride;
+  float state = slot[index];
+  (block - per_span)[index] = state;
+  const int64_t decay = size + (index / ((int64_t)4 * c.dim * tiles)) * c.dim + (index / 4) % c.dim;
+  for (int k = 0; k < spans; ++k, block += per_span) {
+    state = block[decay] * state + block[index];
+    block[index] = state;
+  }
+  slot[index] = state;
 }
 
 template <int R>
 static void launch_keyed_scan(hipStream_t stream, const KeyedScanCall& c) {
-  const int per_token = 4 * 16 * R + 8 * KS_WAVES;
+  const int per_token = (c.form == 0 ? 3 : 2) * 16 * R + 8 * KS_WAVES;
   const int tiles = (c.vdim + 3) / 4, groups = (tiles + KS_WAVES - 1) / KS_WAVES;
+  dim3 block(KS_THREADS);
+  const int span = c.form == 1 ? span_tokens(c.span, c.max_count, c.carry, (int64_t)groups * KS_WAVES * c.heads * c.n_seqs, 1) : 0;
+  if (span > 0 && (int64_t)c.n_seqs * ((c.max_count + span - 1) / span) <= 65535) {
+    KeyedScanCall cut = c;
+    cut.span = span;
+    const int chunk = span < KsRun<R>::MOST ? span : KsRun<R>::MOST;
+    const int spans = (c.max_count + span - 1) / span;
+    dim3 grid(groups, c.heads, c.n_seqs * spans);
+    const size_t lds = (size_t)chunk * per_token * sizeof(float);
+    const int64_t state_floats = (int64_t)c.heads * tiles * c.dim * 4;
+    hipLaunchKernelGGL((keyed_scan_kernel<R, 1, 1>), grid, block, lds, stream, cut, chunk, tiles);
+    hipLaunchKernelGGL(keyed_carry_kernel, dim3((unsigned)((state_floats + 255) / 256), c.n_seqs), dim3(256), 0, stream, cut, tiles);
+    hipLaunchKernelGGL((keyed_scan_kernel<R, 1, 3>), grid, block, lds, stream, cut, chunk, tiles);
+    return;
+  }
   const int chunk = c.tokens < KsRun<R>::MOST ? c.tokens : KsRun<R>::MOST;
-  dim3 grid(groups, c.heads, c.n_seqs), block(KS_THREADS);
+  dim3 grid(groups, c.heads, c.n_seqs);
   const size_t lds = (size_t)chunk * per_token * sizeof(float);
   if (c.form == 0)
-    hipLaunchKernelGGL((keyed_scan_kernel<R, 0>), grid, block, lds, stream, c, chunk, tiles);
+    hipLaunchKernelGGL((keyed_scan_kernel<R, 0, 0>), grid, block, lds, stream, c, chunk, tiles);
   else
-    hipLaunchKernelGGL((keyed_scan_kernel<R, 1>), grid, block, lds, stream, c, chunk, tiles);
+    hipLaunchKernelGGL((keyed_scan_kernel<R, 1, 0>), grid, block, lds, stream, c, chunk, tiles);
 }
 
 BT_EXPORT int bt_keyed_scan_call(void* stream, const KeyedScanCall* c) {

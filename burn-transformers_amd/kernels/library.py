@@ -204,8 +204,9 @@ class KeyedScanCall(ctypes.Structure):
                 ("q", _c_ptr), ("ld_q", _c_i64), ("k", _c_ptr), ("ld_k", _c_i64), ("v", _c_ptr), ("ld_v", _c_i64),
                 ("g", _c_ptr), ("ld_g", _c_i64), ("beta", _c_ptr), ("ld_beta", _c_i64), ("A_log", _c_ptr),
                 ("g_bias", _c_ptr), ("lower", _c_ptr), ("out", _c_ptr), ("ld_out", _c_i64), ("S", _c_ptr),
-                ("state_stride", _c_i64), ("seq_off", _c_ptr), ("slots", _c_ptr)]
-    _step_fields_ = {"tokens": "tokens"}
+                ("state_stride", _c_i64), ("seq_off", _c_ptr), ("slots", _c_ptr), ("span", _c_int), ("max_count", _c_int),
+                ("carry", _c_ptr)]
+    _step_fields_ = {"tokens": "tokens", "max_count": "max_count"}
 
 
 class HeadNormGateCall(ctypes.Structure):
@@ -1302,12 +1303,14 @@ def soft_cap(logits, cap):
 # --- linear attention with a matrix state -------------------------------------------------------
 
 def keyed_scan(q, k, v, g, out, state, step, heads, kv_heads, dim, vdim, form, beta=None, A_log=None, g_bias=None,
-               lower=None, unit=False, unit_eps=1e-6, q_scale=1.0):
+               lower=None, unit=False, unit_eps=1e-6, q_scale=1.0, carry=None):
     """Per head S <- diag(decay) S; S <- S + key u^T; out = S^T query, token after token (csrc/linear_attention.hip).
     ``form`` "delta": u = sigmoid(beta) (v - S^T key), decay = exp(-exp(A_log) g) from step sizes ``g``, ``q`` and
     ``k`` rows of ``kv_heads`` heads (made unit vectors per head with ``unit``, q times ``q_scale``).  ``form``
     "forget": f = lower + (1 - lower) sigmoid(g + g_bias), decay = f, key = 1 - f, query = silu(q), u = v.
-    ``state`` [slots, >= heads * dim * vdim rounded up to 4] float32 is read and left updated."""
+    ``state`` [slots, >= heads * dim * vdim rounded up to 4] float32 is read and left updated.  ``carry``: room from
+    ``scan_carry`` (a slot's state floats, heads * dim extra); with it the "forget" form scans long sequences in
+    spans side by side."""
     _launch(_module("linear_attention"), "bt_keyed_scan_call",
             KeyedScanCall(tokens=v.shape[0], n_seqs=step.n_seqs, heads=heads, kv_heads=kv_heads, dim=dim, vdim=vdim,
                           form={"delta": 0, "forget": 1}[form], unit=1 if unit else 0, unit_eps=unit_eps, q_scale=q_scale,
@@ -1315,7 +1318,8 @@ def keyed_scan(q, k, v, g, out, state, step, heads, kv_heads, dim, vdim, form, b
                           v=v.data_ptr(), ld_v=v.stride(0), g=g.data_ptr(), ld_g=g.stride(0), beta=_ptr(beta),
                           ld_beta=beta.stride(0) if beta is not None else 0, A_log=_ptr(A_log), g_bias=_ptr(g_bias),
                           lower=_ptr(lower), out=out.data_ptr(), ld_out=out.stride(0), S=state.data_ptr(),
-                          state_stride=state.stride(0), seq_off=step.seq_off.data_ptr(), slots=step.slots.data_ptr()))
+                          state_stride=state.stride(0), seq_off=step.seq_off.data_ptr(), slots=step.slots.data_ptr(),
+                          span=SCAN_SPAN if carry is not None else 0, max_count=step.max_count, carry=_ptr(carry)))
 
 
 def head_norm_gate(y, weight, heads, vdim, eps, out, gate=None, mult=1.0):

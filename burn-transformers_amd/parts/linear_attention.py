@@ -135,7 +135,8 @@ class ForgetGateAttention(_MatrixState):
         K.gemm(h, self.in_weight, K.epilogue_f32(fused), packed=self.in_packed)
         y = step.buffer("forget.y", tokens, self.inner, "float32")
         K.keyed_scan(fused[:, :qk], None, fused[:, 2 * qk:], fused[:, qk:2 * qk], y, memory.state(), step, self.heads,
-                     self.heads, self.dim, self.vdim, "forget", g_bias=self.f_bias, lower=self.lower)
+                     self.heads, self.dim, self.vdim, "forget", g_bias=self.f_bias, lower=self.lower,
+                     carry=K.scan_carry(step, self.scan_state, self.heads * self.dim))
         normed = step.buffer("forget.normed", tokens, self.inner_cols, step.dtype)
         K.head_norm_gate(y, self.norm_weight, self.heads, self.vdim, self.eps, normed)
         stream.add_product(step, normed, self.out_weight, packed=self.out_packed)

@@ -36,12 +36,17 @@ def spans_of(lengths, cuts):
     return steps
 
 
-@pytest.mark.parametrize("heads,dim,vdim", [(2, 16, 32), (3, 12, 20), (1, 36, 4), (2, 64, 48), (1, 200, 70), (4, 8, 8)])
-def test_forget_gate_scan_in_portions(heads, dim, vdim):
+@pytest.mark.parametrize("heads,dim,vdim,lengths,cuts,spans", [
+    (2, 16, 32, [150, 7, 66], [1, 3, 64, 65, 130], False), (3, 12, 20, [150, 7, 66], [1, 3, 64, 65, 130], False),
+    (1, 36, 4, [150, 7, 66], [1, 3, 64, 65, 130], False), (2, 64, 48, [150, 7, 66], [1, 3, 64, 65, 130], False),
+    (1, 200, 70, [150, 7, 66], [1, 3, 64, 65, 130], False), (4, 8, 8, [150, 7, 66], [1, 3, 64, 65, 130], False),
+    (2, 16, 32, [700, 40, 330], [5, 505], True), (1, 128, 20, [450, 193, 1], [200], True)])
+def test_forget_gate_scan_in_portions(heads, dim, vdim, lengths, cuts, spans):
     """S <- diag(f) S + (1 - f) v^T, o = S^T silu(q): three sequences in slots of their own, cut into portions of
-    unequal length, down to one token, from the state the last portion left."""
+    unequal length, down to one token, from the state the last portion left; with room for it, long portions are
+    scanned in spans side by side (beside short ones that are not cut, from a state that is not zero)."""
     gen = torch.Generator().manual_seed(heads * 100 + dim)
-    lengths, qk, inner = [150, 7, 66], heads * dim, heads * vdim
+    qk, inner = heads * dim, heads * vdim
     seqs = [torch.randn(n, 2 * qk + inner, generator=gen) for n in lengths]
     f_bias, lower = torch.randn(qk, generator=gen), torch.rand(qk, generator=gen) * 0.9
     want = []
@@ -59,13 +64,15 @@ def test_forget_gate_scan_in_portions(heads, dim, vdim):
     slots = [3, 0, 1]
     state = torch.zeros(4, heads * dim * ((vdim + 3) // 4 * 4), device=DEV)
     got = [torch.zeros(n, inner, dtype=F64) for n in lengths]
-    for step_spans in spans_of(lengths, [1, 3, 64, 65, 130]):
+    for step_spans in spans_of(lengths, cuts):
         step = make_step(torch.float32, [b - a for _, a, b in step_spans], starts=[a for _, a, _ in step_spans],
                          slots=[slots[s] for s, _, _ in step_spans])
         rows = torch.cat([seqs[s][a:b] for s, a, b in step_spans]).to(DEV)
         y = torch.full((rows.shape[0], inner + 2), float("nan"), device=DEV)
+        carry = K.scan_carry(step, state.shape[1], heads * dim) if spans else None
+        assert not spans or step.max_count < 192 or carry is not None
         K.keyed_scan(rows[:, :qk], None, rows[:, 2 * qk:], rows[:, qk:2 * qk], y, state, step, heads, heads, dim, vdim,
-                     "forget", g_bias=f_bias.to(DEV), lower=lower.to(DEV))
+                     "forget", g_bias=f_bias.to(DEV), lower=lower.to(DEV), carry=carry)
         at = 0
         for s, a, b in step_spans:
             got[s][a:b] = y[at:at + b - a, :inner].cpu().double()
