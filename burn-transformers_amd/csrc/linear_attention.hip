@@ -78,10 +78,11 @@ struct KsRun {
 // Decays, queries and keys of a run lie in LDS as planes of [tokens][NP] floats (the forget gate's keys are
 // 1 - decay and have no plane: every wave reads a token's whole row of every plane, and with several waves to a
 // SIMD those reads are what bounds a token's time).  Lane j of the sixteen that share a value channel owns the
-// key channels (16 i + j) V + e, i < R / V, e < V: it reads V neighbouring floats at a time, and neighbouring
-// lanes read neighbouring vectors.
+// key channels j + 16 r, r < R (so the lanes' loads of a register's worth of state are neighbours in memory); in
+// a plane's row channel j + 16 r lies at (16 (r / V) + j) V + r % V, so that a lane reads V neighbouring floats
+// at a time and neighbouring lanes read neighbouring vectors.
 template <int R, int V>
-__device__ __forceinline__ int ks_channel(int sub, int r) { return (16 * (r / V) + sub) * V + r % V; }
+__device__ __forceinline__ int ks_place(int sub, int r) { return (16 * (r / V) + sub) * V + r % V; }
 
 template <int R, int V>
 __device__ __forceinline__ void ks_read(const float* row, int sub, float* out) {
@@ -136,7 +137,7 @@ __global__ void __launch_bounds__(KS_THREADS) keyed_scan_kernel(KeyedScanCall c,
   float S[R], P[R];
 #pragma unroll
   for (int r = 0; r < R; ++r) {
-    const int n = ks_channel<R, V>(sub, r);
+    const int n = sub + 16 * r;
     S[r] = n < c.dim && phase != 1 ? held[(int64_t)n * 4] : 0.f;
     P[r] = 1.0f;
   }
@@ -144,6 +145,7 @@ __global__ void __launch_bounds__(KS_THREADS) keyed_scan_kernel(KeyedScanCall c,
   float* ocol = c.out + head * c.vdim + (live ? p : 0);
   // a thread's entries of a run are key channel `n` of the tokens row0, row0 + ROWS_A_TURN, ...
   const int n = threadIdx.x % NP, row0 = threadIdx.x / NP;
+  const int place = ks_place<R, V>(n % 16, n / 16);       // where channel n lies in a plane's row
   const bool in_head = n < c.dim;
   const int nc = in_head ? n : 0;
   const int col_g = head * c.dim + nc, col_k = shared * c.dim + nc;
@@ -191,9 +193,9 @@ __global__ void __launch_bounds__(KS_THREADS) keyed_scan_kernel(KeyedScanCall c,
             query = PHASE == 1 ? 0.f : silu_f(rq[j]);
           }
         }
-        G[i * NP + n] = decay;
-        if (PHASE != 1) Q[i * NP + n] = query;
-        if (FORM == 0) Kp[i * NP + n] = in_head ? rk[j] : 0.f;
+        G[i * NP + place] = decay;
+        if (PHASE != 1) Q[i * NP + place] = query;
+        if (FORM == 0) Kp[i * NP + place] = in_head ? rk[j] : 0.f;
       }
     }
 #pragma unroll
@@ -218,8 +220,8 @@ __global__ void __launch_bounds__(KS_THREADS) keyed_scan_kernel(KeyedScanCall c,
         const float rq_ = c.q_scale / sqrtf(sum_of_16_lanes(sq) + c.unit_eps);
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-          Kp[i * NP + ks_channel<R, V>(sub, r)] = kk[r] * rk_;
-          Q[i * NP + ks_channel<R, V>(sub, r)] = qq[r] * rq_;
+          Kp[i * NP + ks_place<R, V>(sub, r)] = kk[r] * rk_;
+          Q[i * NP + ks_place<R, V>(sub, r)] = qq[r] * rq_;
         }
       }
       __syncthreads();
@@ -284,7 +286,7 @@ __global__ void __launch_bounds__(KS_THREADS) keyed_scan_kernel(KeyedScanCall c,
   if (!works || phase == 3) return;
 #pragma unroll
   for (int r = 0; r < R; ++r) {
-    const int nn = ks_channel<R, V>(sub, r);
+    const int nn = sub + 16 * r;
     if (nn < c.dim) held[(int64_t)nn * 4] = S[r];
     if (nn < c.dim && phase == 1 && blockIdx.x == 0 && wave == 0 && pl == 0) products[nn] = P[r];
   }
