@@ -247,6 +247,14 @@ class Mixer(Part):
         """Adds the mixer's contribution to ``stream`` (or returns it as a Delta)."""
         raise NotImplementedError
 
+    def ride_along(self, weight, bias=None):
+        """Optional.  A mixer that starts with ONE product of ``h`` that leaves 32-bit sums may take another
+        projection of the same rows along in it (``weight`` [rows, width] in the products' type, ``bias`` float32
+        [rows] or None: a gate that reads what the mixer reads, say) and then returns a function that gives, after
+        ``forward``, the float32 [tokens, rows] results of the step; None (the default): it takes none, and
+        whoever asked runs a product of its own."""
+        return None
+
 
 class FeedForward(Part):
     # True for a feed-forward that hands ``h`` to ``kernels.library.gemm`` and looks at nothing

@@ -97,13 +97,24 @@ class OutputNormBlock(Block):
         for name in ("mixer_norm", "ff_norm"):
             if name in parts and not hasattr(parts[name], "add_output"):
                 raise ValueError(f"output_norm block: {type(parts[name]).__name__} cannot normalise a sublayer's output")
+        # a gate reads what its sublayer reads: where the mixer's first product can take the gate's rows along, it does
+        self.mixer_rider = None
+        gate = parts.get("mixer_gate")
+        if gate is not None and hasattr(gate, "stored") and hasattr(gate, "handed_over"):
+            self.mixer_rider = parts["mixer"].ride_along(gate.stored, gate.bias)
+            if self.mixer_rider is not None:
+                gate.handed_over()
 
     def forward(self, stream, step, memory):
         parts = self.parts
         output = SublayerOutput()
         h = stream.operand(step)
-        gate = {"gate": parts["mixer_gate"].logits(h, step, "block.gate")} if "mixer_gate" in parts else {}
+        gate = {}
+        if "mixer_gate" in parts and self.mixer_rider is None:
+            gate = {"gate": parts["mixer_gate"].logits(h, step, "block.gate")}
         delta = parts["mixer"].forward(h, step, memory, output)
+        if self.mixer_rider is not None:
+            gate = {"gate": self.mixer_rider(step)}
         parts["mixer_norm"].add_output(stream, step, delta if delta is not None else output.take(), self.mult, **gate)
         if "ff" in parts:
             h = stream.operand(step)

@@ -65,6 +65,25 @@ class _MatrixState(Mixer):
         on_gpu = self.in_weight.is_cuda
         self.in_packed = K.PackedWeight(self.in_weight) if on_gpu else None
         self.out_packed = packed_for_stream(self.out_weight) if on_gpu else None
+        self.in_bias, self.fused = None, None
+
+    def ride_along(self, weight, bias=None):
+        if self.in_bias is not None or weight.dtype != self.in_weight.dtype or weight.shape[1] != self.width:
+            return None
+        first, rows = self.fused_cols, weight.shape[0]
+        self.in_weight = torch.cat([self.in_weight, pad_columns(weight, self.in_weight.shape[1])]).contiguous()
+        self.fused_cols = self.in_weight.shape[0]
+        self.in_packed = K.PackedWeight(self.in_weight) if self.in_weight.is_cuda else None
+        self.in_bias = torch.zeros(self.fused_cols, dtype=torch.float32, device=weight.device)
+        if bias is not None:
+            self.in_bias[first:] = bias.float()
+        return lambda step: self.fused[:, first:first + rows]
+
+    def _project(self, h, step, key):
+        """The mixer's first product: every projection of h, and what rides along, as 32-bit sums."""
+        self.fused = step.buffer(key, h.shape[0], self.fused_cols, "float32")
+        K.gemm(h, self.in_weight, K.epilogue_f32(self.fused, self.in_bias), packed=self.in_packed)
+        return self.fused
 
 
 @register("mixer", "gated_delta_rule")
@@ -98,8 +117,7 @@ class GatedDeltaRule(_MatrixState):
         tokens, qk = h.shape[0], self.qk
         rows = memory.state()
         conv_state, scan_state = rows[:, :self.conv_state], rows[:, self.conv_state:]
-        fused = step.buffer("delta.in", tokens, self.fused_cols, "float32")
-        K.gemm(h, self.in_weight, K.epilogue_f32(fused), packed=self.in_packed)
+        fused = self._project(h, step, "delta.in")
         qkv = step.buffer("delta.qkv", tokens, self.channels, "float32")
         K.causal_conv(fused[:, :self.channels], self.conv_weight, None, qkv, conv_state, step)
         dt = step.buffer("delta.dt", tokens, self.heads * self.dim, "float32")
@@ -131,8 +149,7 @@ class ForgetGateAttention(_MatrixState):
 
     def forward(self, h, step, memory, stream):
         tokens, qk = h.shape[0], self.qk
-        fused = step.buffer("forget.in", tokens, self.fused_cols, "float32")
-        K.gemm(h, self.in_weight, K.epilogue_f32(fused), packed=self.in_packed)
+        fused = self._project(h, step, "forget.in")
         y = step.buffer("forget.y", tokens, self.inner, "float32")
         K.keyed_scan(fused[:, :qk], None, fused[:, 2 * qk:], fused[:, qk:2 * qk], y, memory.state(), step, self.heads,
                      self.heads, self.dim, self.vdim, "forget", g_bias=self.f_bias, lower=self.lower,

@@ -41,6 +41,13 @@ class ParallelMixers(Mixer):
     def kernel_modules(self, dtype):
         return tuple(name for _, m, _ in self.sides for name in m.kernel_modules(dtype))
 
+    def ride_along(self, weight, bias=None):
+        for _, mixer, _ in self.sides:
+            rider = mixer.ride_along(weight, bias)
+            if rider is not None:
+                return rider
+        return None
+
     def forward(self, h, step, memory, stream):
         terms = []
         for side, mixer, scale in self.sides:
