@@ -146,3 +146,39 @@ def tolerance(dtype, reference):
     bfloat16 rounds the operands of every product to 8 bits."""
     scale = float(reference.abs().max())
     return 2e-5 + 3e-5 * scale if dtype == "float32" else 3e-2 * scale
+
+
+def random_config(seed):
+    """A configuration drawn from a seed: two to five layers of either kind in any order, with any of the three
+    feed-forwards or none, sizes, windows, taps, parts of the norm and constants from short lists."""
+    import random
+    rng = random.Random(seed)
+    width = rng.choice([64, 96, 128, 160, 256])
+    layers = []
+    for _ in range(rng.randint(2, 5)):
+        if rng.random() < 0.5:
+            mixer = forget(rng.choice([1, 2, 4, 6]), rng.choice([16, 32, 48, 64, 96]), rng.choice([16, 32, 64]))
+        else:
+            kv, dim = rng.choice([1, 2, 4]), rng.choice([16, 32, 48, 64, 80, 128])
+            left = window_attention(kv * rng.choice([1, 2, 3, 4]), kv, dim, rng.choice([16, 32, 48, 64, 128]),
+                                    dim ** -0.5 * rng.choice([0.7, 1.0, 1.5]), rot_dims=rng.choice([0, dim // 4 * 2, dim]),
+                                    base=rng.choice([100.0, 10000.0, 500000.0]),
+                                    window=rng.choice([5, 32, 64, 96, 100, 160]) if rng.random() < 0.85 else None)
+            shared = rng.choice([1, 2, 4])
+            right = delta(shared * rng.choice([1, 2]), shared, rng.choice([16, 32, 64, 128]), rng.choice([16, 32, 64]),
+                          rng.choice([1, 2, 3, 4, 5]), rank=rng.choice([4, 16, 24]))
+            mixer = side_by_side(left, right, rng.choice([0.5, 1.0, 1.2]), rng.choice([0.9, 1.0, 2.0]))
+        kind = rng.random()
+        if kind < 0.15:
+            mlp = None
+        elif kind < 0.45:
+            mlp = dense(rng.choice([64, 200, 256]))
+        else:
+            count, per = rng.choice([1, 2, 4]), rng.choice([1, 2, 3, 4])
+            keep = rng.randint(1, count)
+            grouped = rng.random() < 0.8
+            mlp = moe(count * per, rng.choice([32, 64]), rng.randint(1, keep * per if grouped else count * per),
+                      rng.choice([0.7, 1.5, 7.0]), groups=(count, keep) if grouped else None)
+        layers.append(layer(mixer, mlp))
+    return model_config(layers, width=width, vocab=rng.choice([97, 320, 1000]), groups=rng.choice([g for g in (1, 2, 4, 8) if width % g == 0]),
+                        eps=rng.choice([1e-5, 1e-6]), cap=rng.choice([None, 15.0, 30.0]))

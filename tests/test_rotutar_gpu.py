@@ -9,7 +9,7 @@ pytestmark = pytest.mark.gpu
 import burn_transformers_amd as bt  # noqa: E402
 import plain_rotutar as plain  # noqa: E402
 from burn_transformers_amd.cache.ledger import RELEASED  # noqa: E402
-from rotutar_helpers import (CONFIGS, config_for, engine_for, model_for, plain_logits, prompts_for, tolerance,  # noqa: E402
+from rotutar_helpers import (CONFIGS, config_for, engine_for, random_config, model_for, plain_logits, prompts_for, tolerance,  # noqa: E402
                              weights_for)
 
 DTYPES = ["float32", "bfloat16"]
@@ -218,6 +218,35 @@ def test_a_state_row_that_is_used_again_starts_at_zero():
     got = engine.step([(again, second)], want=[list(range(len(second)))]).clone()
     engine.close(again)
     check(got, plain_logits(name, second), "float32", "a slot used again")
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_configurations_drawn_at_random(seed):
+    """Layers, sizes and constants drawn from a seed, in float32: three unequal prompts in one step, then decoded
+    together while the shorter requests end."""
+    config = random_config(seed)
+    _, tensors = bt.random_tensors(config, seed)
+    stored = {k: v.to(torch.bfloat16) for k, v in tensors.items()}
+    weights = {k: v.float() for k, v in stored.items()}
+    gen = torch.Generator().manual_seed(seed)
+    prompts = [torch.randint(0, config["vocab"], (n,), generator=gen).tolist() for n in (3, 70, 200)]
+    tails = [4, 9, 6]
+    extra = [torch.randint(0, config["vocab"], (t,), generator=gen).tolist() for t in tails]
+    engine = bt.Engine(bt.model_from_tensors(config, stored, "float32", "cuda:0"), max_tokens=1024)
+    slots = [engine.open() for _ in prompts]
+    got = [[] for _ in prompts]
+    logits = engine.step(list(zip(slots, prompts)), want=[list(range(len(p))) for p in prompts])
+    at = 0
+    for i, p in enumerate(prompts):
+        got[i].append(logits[at:at + len(p)].clone())
+        at += len(p)
+    for t in range(max(tails)):
+        live = [i for i in range(len(prompts)) if t < tails[i]]
+        logits = engine.step([(slots[i], [extra[i][t]]) for i in live])
+        for row, i in enumerate(live):
+            got[i].append(logits[row:row + 1].clone())
+    for i, p in enumerate(prompts):
+        check(torch.cat(got[i]), plain.forward(p + extra[i], weights, config), "float32", f"seed {seed} request {i}: {config}")
 
 
 @pytest.mark.parametrize("graphs,programs", [(False, False), (False, True), ("always", True)])
