@@ -1,3 +1,3 @@
-"""Importing this package registers the architectures the library ships (GPT-2, Salopel, Kodatar, Rotutar)."""
+"""Importing this package registers the architectures the library ships (GPT-2, Salopel, Kodatar, Rotutar, Gavasun)."""
 
-from . import gpt2, kodatar, rotutar, salopel  # noqa: F401
+from . import gavasun, gpt2, kodatar, rotutar, salopel  # noqa: F401

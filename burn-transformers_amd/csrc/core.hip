@@ -466,12 +466,14 @@ BT_EXPORT int bt_gemm_plain(void* stream, int dtype, const void* A, int64_t lda,
 // Keys beyond the token's own position are never read.
 // ---------------------------------------------------------------------------------------------
 #define PLAIN_CHUNK 1024
+#define PLAIN_MAX_HEAD 768                    // a thread keeps up to three output channels
+#define PLAIN_PER_THREAD (PLAIN_MAX_HEAD / 256)
 
 
 template <typename T>
 __global__ void __launch_bounds__(256)
 attention_plain_kernel(AttnArgs a) {
-  __shared__ float qs[256];
+  __shared__ float qs[PLAIN_MAX_HEAD];
   __shared__ float ps[PLAIN_CHUNK];
   __shared__ float scratch[32];
   int t = blockIdx.x, head = blockIdx.y;
@@ -483,7 +485,10 @@ attention_plain_kernel(AttnArgs a) {
   for (int c = threadIdx.x; c < hd; c += blockDim.x) qs[c] = to_float(q[c]);
   __syncthreads();
   int lo = bt_first_seen(pos, a.window, a.chunk);
-  float run_max = -INFINITY, run_sum = 0.f, acc = 0.f;  // acc: channel threadIdx.x (< hd)
+  float run_max = -INFINITY, run_sum = 0.f;
+  float acc[PLAIN_PER_THREAD];                          // channels threadIdx.x, threadIdx.x + 256, ... (< hd)
+#pragma unroll
+  for (int j = 0; j < PLAIN_PER_THREAD; ++j) acc[j] = 0.f;
   const T* keys = static_cast<const T*>(a.kv.keys);
   const T* values = static_cast<const T*>(a.kv.values);
   for (int c0 = lo; c0 <= pos; c0 += PLAIN_CHUNK) {
@@ -512,26 +517,33 @@ attention_plain_kernel(AttnArgs a) {
     run_sum = run_sum * rescale + chunk_sum;
     run_max = new_max;
     __syncthreads();
-    if ((int)threadIdx.x < hd) {
-      acc *= rescale;
+#pragma unroll
+    for (int j = 0; j < PLAIN_PER_THREAD; ++j) {
+      const int channel = threadIdx.x + 256 * j;
+      if (channel >= hd) break;
+      acc[j] *= rescale;
       for (int i = 0; i < n; ++i) {
         int k = c0 + i;
         const T* vr = values + kv_block_base(a.kv, seq, k, kv_head);
-        acc = fmaf(ps[i], to_float(vr[value_offset(hd, k, threadIdx.x)]), acc);
+        acc[j] = fmaf(ps[i], to_float(vr[value_offset(hd, k, channel)]), acc[j]);
       }
     }
     __syncthreads();
   }
   run_sum += bt_sink_term(a.sink, head, run_max);
-  if ((int)threadIdx.x < hd) {
-    T* o = static_cast<T*>(a.out) + (int64_t)t * a.ldo + head * hd;
-    o[threadIdx.x] = from_float<T>(run_sum > 0.f ? acc / run_sum : 0.f);
+  T* o = static_cast<T*>(a.out) + (int64_t)t * a.ldo + head * hd;
+#pragma unroll
+  for (int j = 0; j < PLAIN_PER_THREAD; ++j) {
+    const int channel = threadIdx.x + 256 * j;
+    if (channel < hd) o[channel] = from_float<T>(run_sum > 0.f ? acc[j] / run_sum : 0.f);
   }
 }
 
 int bt_check_attention(const AttnArgs& a, const char* who) {
   int hd = a.kv.head_dim;
-  if (hd <= 0 || hd > 256) BT_REFUSE("%s: head size %d outside 1..256 (a work-group holds a query and one channel per thread)", who, hd);
+  if (hd <= 0 || hd > PLAIN_MAX_HEAD)
+    BT_REFUSE("%s: head size %d outside 1..%d (a work-group holds a query and up to %d channels per thread)", who, hd,
+              PLAIN_MAX_HEAD, PLAIN_PER_THREAD);
   if (a.kv.kv_heads <= 0 || a.q_heads <= 0 || a.q_heads % a.kv.kv_heads != 0)
     BT_REFUSE("%s: %d query heads cannot share %d key/value heads", who, a.q_heads, a.kv.kv_heads);
   if (a.window < 0 || a.chunk < 0) BT_REFUSE("%s: window %d and chunk %d must not be negative", who, a.window, a.chunk);

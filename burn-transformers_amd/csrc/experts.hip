@@ -239,10 +239,16 @@ struct GatedExpertsCall {
   const void* h;            // [tokens][ldh]: the experts' input (read for identity experts only)
   int64_t ldh;
   float* identity_out;      // [tokens][width] float32: (sum of the identity experts' weights) * h; or null
-  int act;                  // 0: silu(g) * u; 1: min(g, limit) * sigmoid(alpha * min(g, limit)) * (clamp(u, -limit, limit) + 1)
+  int act;                  // 0: silu(g) * u; 1: min(g, limit) * sigmoid(alpha * min(g, limit)) * (clamp(u, -limit, limit) + 1);
+                            // 2, 3: units WITHOUT a gate, gelu(u) in its exact (erf) form and silu(u): `gu` then holds per
+                            // expert its ff up rows only, the shared expert's behind them
   float limit;
   float alpha;
 };
+
+__device__ __forceinline__ float plain_unit(const GatedExpertsCall& c, float u) {
+  return c.act == 2 ? 0.5f * u * (1.0f + erff(u * 0.70710678118654752f)) : u / (1.0f + expf(-u));
+}
 
 __device__ __forceinline__ float gated_unit(const GatedExpertsCall& c, float g, float u) {
   if (c.act == 1) {
@@ -260,20 +266,28 @@ __global__ void __launch_bounds__(256) gated_experts_kernel(GatedExpertsCall c) 
   T* hidden = static_cast<T*>(c.hidden) + (int64_t)t * c.ld_hidden;
   const float* weights = c.weights + (int64_t)t * (c.experts + c.identity);
   const int routed = c.experts * c.ff;
+  const bool gated = c.act < 2;
   // a token's columns are dealt to the work-groups of its row of the grid (a decode step has few tokens)
   for (int col = blockIdx.y * blockDim.x + threadIdx.x; col < c.hidden_cols; col += gridDim.y * blockDim.x) {
     float out = 0.f;
     if (col < routed) {
       const int e = col / c.ff, i = col - e * c.ff;
       const float w = weights[e];
-      if (w != 0.f) {
+      if (w != 0.f && gated) {
         const float g = to_float(gu[(int64_t)e * 2 * c.ff + i]), u = to_float(gu[(int64_t)e * 2 * c.ff + c.ff + i]);
         out = w * gated_unit(c, g, u);
+      } else if (w != 0.f) {
+        out = w * plain_unit(c, to_float(gu[col]));
       }
     } else if (col < routed + c.shared_ff) {
       const int i = col - routed;
-      const float g = to_float(gu[(int64_t)2 * routed + i]), u = to_float(gu[(int64_t)2 * routed + c.shared_ff + i]);
-      out = (c.gate ? c.gate[t] : 1.0f) * gated_unit(c, g, u);
+      const float share = c.gate ? c.gate[t] : 1.0f;
+      if (gated) {
+        const float g = to_float(gu[(int64_t)2 * routed + i]), u = to_float(gu[(int64_t)2 * routed + c.shared_ff + i]);
+        out = share * gated_unit(c, g, u);
+      } else {
+        out = share * plain_unit(c, to_float(gu[col]));
+      }
     }
     hidden[col] = from_float<T>(out);
   }
@@ -291,9 +305,9 @@ BT_EXPORT int bt_gated_experts_call(void* stream, const GatedExpertsCall* c) {
   if (c->experts < 0 || c->ff <= 0 || c->shared_ff < 0 || c->identity < 0)
     BT_REFUSE("gated_experts: %d experts of %d, a shared one of %d and %d identity experts", c->experts, c->ff, c->shared_ff, c->identity);
   const int64_t columns = (int64_t)c->experts * c->ff + c->shared_ff;
-  if (c->hidden_cols < columns || c->ld_hidden < c->hidden_cols || c->ld_gu < 2 * columns)
+  if (c->act < 0 || c->act > 3) BT_REFUSE("gated_experts: unknown activation %d", c->act);
+  if (c->hidden_cols < columns || c->ld_hidden < c->hidden_cols || c->ld_gu < (c->act < 2 ? 2 : 1) * columns)
     BT_REFUSE("gated_experts: the rows do not hold the experts");
-  if (c->act != 0 && c->act != 1) BT_REFUSE("gated_experts: unknown activation %d", c->act);
   if (!c->gu || (!c->weights && c->experts + c->identity > 0) || !c->hidden || (c->identity_out && (!c->h || c->width <= 0)))
     BT_REFUSE("gated_experts: missing operand");
   // about 1,024 columns a work-group, fewer work-groups a token where there are many tokens

@@ -2,7 +2,12 @@
 // latents; only the key/value latent is cached, and attention runs on it directly).
 //   * latent norms: the two RMS norms behind the fused down-projection; the query latent goes to a
 //     buffer for the next product, the key/value latent straight into the paged cache, where it is
-//     the one shared "head" whose keys and values are the same vector
+//     the one shared "head" whose keys and values are the same vector.  With `rot_dim` > 0 the down-projection
+//     has that many more rows behind the key/value latent: one key part that all heads share, not normalised,
+//     turned by the token's position (channel 2 i with channel 2 i + 1, or i with i + rot_dim / 2), kept behind
+//     the latent in the cached head's KEYS (its values have zeros there)
+//   * query rotation: the absorbed queries (32-bit sums, a head's latent part and behind it its turned part)
+//     into the attention kernels' type, the turned part rotated by the token's position
 //   * head projection with gate: per head out = sigmoid(g) * (W_h . ctx_h), the value up-projection
 //     applied AFTER the weighted sum over positions (it is linear, so it commutes with the sum)
 // Statistics and sums are 32-bit.
@@ -23,7 +28,11 @@ struct LatentNormCall {
   int64_t ld_q;
   const int* tok_seq;
   const int* tok_pos;
-  KvView kv;              // one head of head_dim >= kv_rank
+  KvView kv;              // one head of head_dim >= kv_rank + rot_dim
+  int rot_dim;            // channels of the shared turned key part (even; 0: none), at in[kv_offset + kv_rank ..]
+  int pairing;            // 0: channel i turns with channel i + rot_dim / 2; 1: channel 2 i with channel 2 i + 1
+  float amplitude;        // factor on every sine and cosine
+  const float* inv_freq;  // [rot_dim / 2]
 };
 
 template <typename T>
@@ -46,10 +55,21 @@ __global__ void __launch_bounds__(256) latent_norm_kernel(LatentNormCall c) {
     const int64_t base = kv_block_base(c.kv, seq, pos, 0);
     T* keys = static_cast<T*>(c.kv.keys) + base;
     T* values = static_cast<T*>(c.kv.values) + base;
+    const int half = c.rot_dim >> 1;
     for (int col = threadIdx.x; col < hd; col += blockDim.x) {
       const T v = from_float<T>(col < n ? row[col] * rstd * gamma[col] : 0.f);
-      keys[key_offset(hd, pos, col)] = v;
+      if (col < n || col >= n + c.rot_dim) keys[key_offset(hd, pos, col)] = v;
       values[value_offset(hd, pos, col)] = v;
+    }
+    for (int i = threadIdx.x; i < half; i += blockDim.x) {
+      float sn, cs;
+      sincosf((float)pos * c.inv_freq[i], &sn, &cs);
+      sn *= c.amplitude;
+      cs *= c.amplitude;
+      const int first = c.pairing == 1 ? 2 * i : i, second = c.pairing == 1 ? 2 * i + 1 : i + half;
+      const float u = row[n + first], w = row[n + second];
+      keys[key_offset(hd, pos, n + first)] = from_float<T>(u * cs - w * sn);
+      keys[key_offset(hd, pos, n + second)] = from_float<T>(w * cs + u * sn);
     }
   }
 }
@@ -57,10 +77,12 @@ __global__ void __launch_bounds__(256) latent_norm_kernel(LatentNormCall c) {
 BT_EXPORT int bt_latent_norm_call(void* stream, const LatentNormCall* c) {
   if (c->tokens <= 0) return BT_OK;
   if (c->q_rank <= 0 || c->kv_rank <= 0) BT_REFUSE("latent_norm: ranks %d and %d must be positive", c->q_rank, c->kv_rank);
-  if (c->kv.kv_heads != 1 || c->kv.head_dim < c->kv_rank)
+  if (c->rot_dim < 0 || c->rot_dim % 2 != 0 || (c->pairing != 0 && c->pairing != 1) || (c->rot_dim > 0 && !c->inv_freq))
+    BT_REFUSE("latent_norm: a turned key part of %d channels (even, with frequencies), pairing %d (0 or 1)", c->rot_dim, c->pairing);
+  if (c->kv.kv_heads != 1 || c->kv.head_dim < c->kv_rank + c->rot_dim)
     BT_REFUSE("latent_norm: the cache keeps %d heads of %d, expected one of at least %d", c->kv.kv_heads,
-              c->kv.head_dim, c->kv_rank);
-  if (c->q_cols < c->q_rank || c->ld_q < c->q_cols || c->ld < c->kv_offset + c->kv_rank || c->kv_offset < c->q_rank)
+              c->kv.head_dim, c->kv_rank + c->rot_dim);
+  if (c->q_cols < c->q_rank || c->ld_q < c->q_cols || c->ld < c->kv_offset + c->kv_rank + c->rot_dim || c->kv_offset < c->q_rank)
     BT_REFUSE("latent_norm: the rows do not hold the latents");
   if (!c->in || !c->q_gamma || !c->kv_gamma || !c->q_out || !c->tok_seq || !c->tok_pos || !c->kv.blocks ||
       !c->kv.keys || !c->kv.values)
@@ -71,6 +93,64 @@ BT_EXPORT int bt_latent_norm_call(void* stream, const LatentNormCall* c) {
   else
     hipLaunchKernelGGL(latent_norm_kernel<bf16_t>, grid, block, 0, (hipStream_t)stream, *c);
   return bt_check_launch("latent_norm");
+}
+
+// q[t][h * pitch + j] = in[t][h * pitch + j], the channels [rot_at, rot_at + rot_dim) of every head turned by the
+// token's position: pairs (2 i, 2 i + 1) or (i, i + rot_dim / 2) of that range, by the angle position * inv_freq[i].
+struct LatentQueryCall {
+  int dtype;              // element type of `out`: 0 float32, 1 bfloat16
+  int tokens, heads;
+  int pitch;              // channels of a head in `in` and `out`
+  int rot_at, rot_dim;    // the turned range inside a head
+  int pairing;
+  float amplitude;
+  const float* in;        // [tokens][ld_in] float32
+  int64_t ld_in;
+  void* out;              // [tokens][ld_out]
+  int64_t ld_out;
+  const float* inv_freq;  // [rot_dim / 2]
+  const int* tok_pos;
+};
+
+template <typename T>
+__global__ void __launch_bounds__(256) latent_query_kernel(LatentQueryCall c) {
+  const int t = blockIdx.x, pos = c.tok_pos[t], half = c.rot_dim >> 1;
+  const float* in = c.in + (int64_t)t * c.ld_in;
+  T* out = static_cast<T*>(c.out) + (int64_t)t * c.ld_out;
+  const int columns = c.heads * c.pitch;
+  for (int col = blockIdx.y * blockDim.x + threadIdx.x; col < columns; col += gridDim.y * blockDim.x) {
+    const int head = col / c.pitch, j = col - head * c.pitch - c.rot_at;
+    float v = in[col];
+    if (j >= 0 && j < c.rot_dim) {
+      // channel j of the turned range: the first of its pair takes u cos - v sin, the second v cos + u sin
+      const int i = c.pairing == 1 ? j >> 1 : (j < half ? j : j - half);
+      const bool second = c.pairing == 1 ? (j & 1) : j >= half;
+      const int mate = c.pairing == 1 ? (j ^ 1) : (second ? j - half : j + half);
+      const float other = in[col - j + mate];
+      float sn, cs;
+      sincosf((float)pos * c.inv_freq[i], &sn, &cs);
+      v = c.amplitude * (second ? v * cs + other * sn : v * cs - other * sn);
+    }
+    out[col] = from_float<T>(v);
+  }
+}
+
+BT_EXPORT int bt_latent_query_call(void* stream, const LatentQueryCall* c) {
+  if (c->tokens <= 0) return BT_OK;
+  if (c->heads <= 0 || c->pitch <= 0 || c->rot_at < 0 || c->rot_dim < 0 || c->rot_dim % 2 != 0 || c->rot_at + c->rot_dim > c->pitch)
+    BT_REFUSE("latent_query: %d heads of %d with a turned range of %d from %d", c->heads, c->pitch, c->rot_dim, c->rot_at);
+  if (c->pairing != 0 && c->pairing != 1) BT_REFUSE("latent_query: pairing %d must be 0 or 1", c->pairing);
+  const int64_t columns = (int64_t)c->heads * c->pitch;
+  if (!c->in || !c->out || !c->tok_pos || (c->rot_dim > 0 && !c->inv_freq) || c->ld_in < columns || c->ld_out < columns)
+    BT_REFUSE("latent_query: missing operand or rows too short");
+  int per_token = (int)((columns + 1023) / 1024);
+  if (per_token > 64) per_token = 64;
+  dim3 grid(c->tokens, per_token), block(256);
+  if (c->dtype == 0)
+    hipLaunchKernelGGL(latent_query_kernel<float>, grid, block, 0, (hipStream_t)stream, *c);
+  else
+    hipLaunchKernelGGL(latent_query_kernel<bf16_t>, grid, block, 0, (hipStream_t)stream, *c);
+  return bt_check_launch("latent_query");
 }
 
 // out[t][h * vdim + v] = sigmoid(gate[t][h * vdim + v]) * sum_r W[h * vdim + v][r] * ctx[t][h * ld_head + r]

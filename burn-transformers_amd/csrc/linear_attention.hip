@@ -8,7 +8,8 @@
 //     How g, k and q come about is the kernel's `form`:
 //       form 0 (gated delta rule): q and k are rows of their own (heads may share them), optionally made unit
 //           vectors per head here, x / sqrt(sum x^2 + unit_eps), q times q_scale; g = exp(-exp(A_log[head]) * dt)
-//           from step sizes dt per head and key channel; beta = sigmoid(beta logit of the head)
+//           from step sizes dt per head and key channel, or one per head for all its key channels (`decay_span` 1);
+//           with `dt_bias` the step sizes come raw and dt = softplus(raw + dt_bias); beta = sigmoid(beta logit of the head)
 //       form 1 (forget gate that also decides what is written): f = lower + (1 - lower) * sigmoid(f_raw + f_bias)
 //           per head and key channel; g = f, k = 1 - f, q = silu(q_raw); no beta
 //   * head norm with a gate: every head's read-out over its root mean square over vdim, times a scale of
@@ -33,8 +34,9 @@ struct KeyedScanCall {
   int64_t ld_k;
   const float* v;         // [tokens][ld_v]: head h at columns h * vdim
   int64_t ld_v;
-  const float* g;         // [tokens][ld_g]: head h at columns h * dim: step sizes (form 0), gate logits (form 1)
-  int64_t ld_g;
+  const float* g;         // [tokens][ld_g]: head h at columns h * dim: step sizes (form 0), gate logits (form 1);
+  int64_t ld_g;           // with decay_span 1 head h at column h
+
   const float* beta;      // [tokens][ld_beta]: one logit a head (form 0)
   int64_t ld_beta;
   const float* A_log;     // [heads] (form 0)
@@ -54,6 +56,8 @@ struct KeyedScanCall {
   int span;
   int max_count;
   float* carry;
+  int decay_span;         // form 0: 0 a step size per head and key channel, 1 one per head
+  const float* dt_bias;   // form 0: null, or [heads * dim] ([heads] with decay_span 1): g holds raw sums, dt = softplus(g + dt_bias)
 };
 
 // One wave per (4 value channels of a head, sequence): sixteen lanes share a channel, each owns R key channels
@@ -148,12 +152,14 @@ __global__ void __launch_bounds__(KS_THREADS) keyed_scan_kernel(KeyedScanCall c,
   const int place = ks_place<R, V>(n % 16, n / 16);       // where channel n lies in a plane's row
   const bool in_head = n < c.dim;
   const int nc = in_head ? n : 0;
-  const int col_g = head * c.dim + nc, col_k = shared * c.dim + nc;
+  const int col_g = FORM == 0 && c.decay_span == 1 ? head : head * c.dim + nc, col_k = shared * c.dim + nc;
   float low = 0.f, bias = 0.f;
   if (FORM == 1) {
     low = c.lower[col_g];
     bias = c.g_bias ? c.g_bias[col_g] : 0.f;
   }
+  const bool raw_steps = FORM == 0 && c.dt_bias != nullptr;
+  if (raw_steps) bias = c.dt_bias[col_g];
   const int ch = tile * 4 + (lane & 3);                   // the value channel of a lane's (v, beta) pairs
   const int chc = ch < c.vdim ? ch : 0;
   float rg[KS_LOADS], rk[KS_LOADS], rq[KS_LOADS], rv[TOK_LOADS], rb[TOK_LOADS];
@@ -186,7 +192,7 @@ __global__ void __launch_bounds__(KS_THREADS) keyed_scan_kernel(KeyedScanCall c,
         float decay = 0.f, query = 0.f;
         if (in_head) {
           if (FORM == 0) {
-            decay = expf(rate * rg[j]);
+            decay = expf(rate * (raw_steps ? softplus_f(rg[j] + bias) : rg[j]));
             query = rq[j];
           } else {
             decay = low + (1.0f - low) / (1.0f + expf(-(rg[j] + bias)));
@@ -353,7 +359,8 @@ BT_EXPORT int bt_keyed_scan_call(void* stream, const KeyedScanCall* c) {
   if (c->form == 0 && (!c->k || !c->beta || !c->A_log)) BT_REFUSE("keyed_scan: the delta rule lacks keys, beta or A_log");
   if (c->form == 1 && !c->lower) BT_REFUSE("keyed_scan: the forget gate lacks its lower bound");
   const int64_t qk = (int64_t)(c->form == 0 ? c->kv_heads : c->heads) * c->dim;
-  if (c->ld_q < qk || (c->form == 0 && c->ld_k < qk) || c->ld_g < (int64_t)c->heads * c->dim ||
+  if (c->decay_span != 0 && (c->decay_span != 1 || c->form != 0)) BT_REFUSE("keyed_scan: a decay per head goes with the delta rule");
+  if (c->ld_q < qk || (c->form == 0 && c->ld_k < qk) || c->ld_g < (int64_t)c->heads * (c->decay_span == 1 ? 1 : c->dim) ||
       c->ld_v < (int64_t)c->heads * c->vdim || c->ld_out < (int64_t)c->heads * c->vdim ||
       (c->form == 0 && c->ld_beta < c->heads))
     BT_REFUSE("keyed_scan: rows too short for %d heads of %d and %d", c->heads, c->dim, c->vdim);
@@ -386,6 +393,7 @@ struct HeadNormGateCall {
   const float* weight;    // [vdim]
   void* out;              // [tokens][ld_out]
   int64_t ld_out;
+  int gate_act;           // what the gate's logits z become: 0 sigmoid(z), 1 silu(z) = z sigmoid(z)
 };
 
 template <typename T>
@@ -399,7 +407,10 @@ __global__ void __launch_bounds__(256) head_norm_gate_kernel(HeadNormGateCall c)
     const float scale = c.mult / sqrtf(wave_sum(squares) / (float)c.vdim + c.eps);
     for (int i = lane; i < c.vdim; i += 64) {
       float v = y[i] * scale * c.weight[i];
-      if (c.gate) v *= 1.0f / (1.0f + expf(-c.gate[(int64_t)t * c.ld_gate + head * c.vdim + i]));
+      if (c.gate) {
+        const float z = c.gate[(int64_t)t * c.ld_gate + head * c.vdim + i];
+        v *= (c.gate_act == 1 ? z : 1.0f) / (1.0f + expf(-z));
+      }
       out[head * c.vdim + i] = from_float<T>(v);
     }
   }
@@ -414,6 +425,7 @@ BT_EXPORT int bt_head_norm_gate_call(void* stream, const HeadNormGateCall* c) {
   if (!c->y || !c->weight || !c->out || c->ld_y < columns || c->out_cols < columns || c->ld_out < c->out_cols ||
       (c->gate && c->ld_gate < columns))
     BT_REFUSE("head_norm_gate: missing operand or rows too short");
+  if (c->gate_act != 0 && c->gate_act != 1) BT_REFUSE("head_norm_gate: unknown activation %d of the gate", c->gate_act);
   int per_token = (c->heads + 3) / 4;
   if (per_token > 64) per_token = 64;
   dim3 grid(c->tokens, per_token), block(256);

@@ -7,7 +7,8 @@
 //     sizes; the cache keeps heads of one size, and what lies behind a head's own channels is zero.
 // Channel i < rot_dims / 2 is paired with channel i + rot_dims / 2 (`pairing` 0, the halves) or channel
 // 2 i with channel 2 i + 1 (`pairing` 1, neighbours); the pair (u, v) at position p
-// becomes (u cos a - v sin a, v cos a + u sin a), a = p * inv_freq[i].  With `norm_span` 1 the root mean
+// becomes (u cos a - v sin a, v cos a + u sin a), a = p * inv_freq[i], sine and cosine times `amplitude`
+// (one where the frequencies are not rescaled; schedules that slow long waves let both grow a little).  With `norm_span` 1 the root mean
 // square is taken over a token's WHOLE query (or key) projection, all heads at once, and the scale has
 // an entry for every channel of the projection.  The frequencies come as a
 // table, so any schedule of them (scaled, interpolated) is the caller's.  Norms, angles and the
@@ -33,6 +34,7 @@ struct HeadRotaryCall {
   KvView kv;              // kv_heads heads of head_dim >= max(dim, vdim)
   int pairing;            // 0: channel i turns with channel i + rot_dims / 2; 1: channel 2 i with channel 2 i + 1
   int norm_span;          // 0: every head over its own root mean square; 1: the whole projection over one
+  float amplitude;        // factor on every sine and cosine
 };
 
 #define HR_WAVES 4
@@ -101,6 +103,8 @@ __global__ void __launch_bounds__(HR_WAVES * 64) head_rotary_kernel(HeadRotaryCa
     for (int i = lane; i < half; i += 64) {
       float sn, cs;
       sincosf((float)pos * c.inv_freq[i], &sn, &cs);
+      sn *= c.amplitude;
+      cs *= c.amplitude;
       const int first = c.pairing == 1 ? 2 * i : i, second = c.pairing == 1 ? 2 * i + 1 : i + half;
       const float u = row[first], v = row[second];
       store(first, u * cs - v * sn);

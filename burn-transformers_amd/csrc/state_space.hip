@@ -75,6 +75,7 @@ struct CausalConvCall {
   const int* tok_seq;
   const int* seq_off;     // [n_seqs + 1]
   const int* slots;       // [n_seqs]
+  int act;                // what follows the sum: 0 silu, 1 nothing
 };
 
 // SHIFT: every sequence of the step brings one token (a decode step), so a (sequence, channel) pair
@@ -99,7 +100,7 @@ __global__ void __launch_bounds__(256) causal_conv_kernel(CausalConvCall c) {
                              : held[(int64_t)(c.taps - 1 + src) * c.channels + ch];
     sum = fmaf(c.weight[(int64_t)ch * c.taps + j], u, sum);
   }
-  const float y = silu_f(sum);
+  const float y = c.act == 0 ? silu_f(sum) : sum;
   c.out[(int64_t)t * c.ld_out + ch] = y;
   if (cast) cast[(int64_t)t * c.ld_cast + ch] = from_float<T>(y);
   if (SHIFT) {
@@ -129,6 +130,7 @@ BT_EXPORT int bt_causal_conv_call(void* stream, const CausalConvCall* c) {
     BT_REFUSE("causal_conv: %d channels, %d taps, %d sequences: all must be positive", c->channels, c->taps, c->n_seqs);
   if (!c->in || !c->weight || !c->out || !c->tok_seq || !c->seq_off || !c->slots || (c->taps > 1 && !c->state))
     BT_REFUSE("causal_conv: missing operand");
+  if (c->act != 0 && c->act != 1) BT_REFUSE("causal_conv: unknown activation %d", c->act);
   if (c->ld_in < c->channels || c->ld_out < c->channels || (c->cast && (c->cast_cols < c->channels || c->ld_cast < c->cast_cols)))
     BT_REFUSE("causal_conv: the rows do not hold %d channels", c->channels);
   if (c->taps > 1 && c->state_stride < (int64_t)(c->taps - 1) * c->channels)

@@ -110,7 +110,14 @@ class LatentNormCall(ctypes.Structure):
     _fields_ = [("dtype", _c_int), ("tokens", _c_int), ("q_rank", _c_int), ("q_cols", _c_int), ("kv_rank", _c_int),
                 ("kv_offset", _c_int), ("eps", _c_float), ("input", _c_ptr), ("ld", _c_i64), ("q_gamma", _c_ptr),
                 ("kv_gamma", _c_ptr), ("q_out", _c_ptr), ("ld_q", _c_i64), ("tok_seq", _c_ptr), ("tok_pos", _c_ptr),
-                ("kv", KvView)]
+                ("kv", KvView), ("rot_dim", _c_int), ("pairing", _c_int), ("amplitude", _c_float), ("inv_freq", _c_ptr)]
+    _step_fields_ = {"tokens": "tokens"}
+
+
+class LatentQueryCall(ctypes.Structure):
+    _fields_ = [("dtype", _c_int), ("tokens", _c_int), ("heads", _c_int), ("pitch", _c_int), ("rot_at", _c_int),
+                ("rot_dim", _c_int), ("pairing", _c_int), ("amplitude", _c_float), ("input", _c_ptr), ("ld_in", _c_i64),
+                ("out", _c_ptr), ("ld_out", _c_i64), ("inv_freq", _c_ptr), ("tok_pos", _c_ptr)]
     _step_fields_ = {"tokens": "tokens"}
 
 
@@ -125,7 +132,7 @@ class CausalConvCall(ctypes.Structure):
     _fields_ = [("cast_dtype", _c_int), ("tokens", _c_int), ("n_seqs", _c_int), ("channels", _c_int), ("taps", _c_int),
                 ("cast_cols", _c_int), ("input", _c_ptr), ("ld_in", _c_i64), ("weight", _c_ptr), ("bias", _c_ptr),
                 ("out", _c_ptr), ("ld_out", _c_i64), ("cast", _c_ptr), ("ld_cast", _c_i64), ("state", _c_ptr),
-                ("state_stride", _c_i64), ("tok_seq", _c_ptr), ("seq_off", _c_ptr), ("slots", _c_ptr)]
+                ("state_stride", _c_i64), ("tok_seq", _c_ptr), ("seq_off", _c_ptr), ("slots", _c_ptr), ("act", _c_int)]
     _step_fields_ = {"tokens": "tokens"}
 
 
@@ -164,7 +171,8 @@ class HeadRotaryCall(ctypes.Structure):
     _fields_ = [("dtype", _c_int), ("tokens", _c_int), ("heads", _c_int), ("kv_heads", _c_int), ("dim", _c_int),
                 ("vdim", _c_int), ("rot_dims", _c_int), ("eps", _c_float), ("input", _c_ptr), ("ld", _c_i64),
                 ("q_gamma", _c_ptr), ("k_gamma", _c_ptr), ("inv_freq", _c_ptr), ("q_out", _c_ptr), ("ld_q", _c_i64),
-                ("tok_seq", _c_ptr), ("tok_pos", _c_ptr), ("kv", KvView), ("pairing", _c_int), ("norm_span", _c_int)]
+                ("tok_seq", _c_ptr), ("tok_pos", _c_ptr), ("kv", KvView), ("pairing", _c_int), ("norm_span", _c_int),
+                ("amplitude", _c_float)]
     _step_fields_ = {"tokens": "tokens"}
 
 
@@ -205,14 +213,14 @@ class KeyedScanCall(ctypes.Structure):
                 ("g", _c_ptr), ("ld_g", _c_i64), ("beta", _c_ptr), ("ld_beta", _c_i64), ("A_log", _c_ptr),
                 ("g_bias", _c_ptr), ("lower", _c_ptr), ("out", _c_ptr), ("ld_out", _c_i64), ("S", _c_ptr),
                 ("state_stride", _c_i64), ("seq_off", _c_ptr), ("slots", _c_ptr), ("span", _c_int), ("max_count", _c_int),
-                ("carry", _c_ptr)]
+                ("carry", _c_ptr), ("decay_span", _c_int), ("dt_bias", _c_ptr)]
     _step_fields_ = {"tokens": "tokens", "max_count": "max_count"}
 
 
 class HeadNormGateCall(ctypes.Structure):
     _fields_ = [("out_dtype", _c_int), ("tokens", _c_int), ("heads", _c_int), ("vdim", _c_int), ("out_cols", _c_int),
                 ("eps", _c_float), ("mult", _c_float), ("y", _c_ptr), ("ld_y", _c_i64), ("gate", _c_ptr),
-                ("ld_gate", _c_i64), ("weight", _c_ptr), ("out", _c_ptr), ("ld_out", _c_i64)]
+                ("ld_gate", _c_i64), ("weight", _c_ptr), ("out", _c_ptr), ("ld_out", _c_i64), ("gate_act", _c_int)]
     _step_fields_ = {"tokens": "tokens"}
 
 
@@ -1098,15 +1106,30 @@ def poly_norm(z, columns, coefficients, eps, out):
 
 # --- latent attention ------------------------------------------------------------------------
 
-def latent_norm(fused, q_rank, kv_offset, kv_rank, q_gamma, kv_gamma, eps, q_out, tok_seq, tok_pos, kv_view, dtype):
+def latent_norm(fused, q_rank, kv_offset, kv_rank, q_gamma, kv_gamma, eps, q_out, tok_seq, tok_pos, kv_view, dtype,
+                rot_dim=0, inv_freq=None, neighbours=True, amplitude=1.0):
     """The two RMS norms behind a fused down-projection (float32 rows ``fused``): columns [0, q_rank)
     go normalised to ``q_out`` (zeros behind them), columns [kv_offset, kv_offset + kv_rank) into the
-    paged cache at each token's position, as the keys AND the values of its one head."""
+    paged cache at each token's position, as the keys AND the values of its one head.  With ``rot_dim`` the
+    next so many columns are a key part that is not normalised but turned by the token's position (angles
+    position * ``inv_freq[i]``, sine and cosine times ``amplitude``; channel 2 i with 2 i + 1, or with
+    ``neighbours`` False i with i + rot_dim / 2) and kept behind the latent in the head's keys."""
     _launch(_module("latent"), "bt_latent_norm_call",
             LatentNormCall(dtype=DTYPE_CODES[dtype], tokens=fused.shape[0], q_rank=q_rank, q_cols=q_out.shape[1],
                            kv_rank=kv_rank, kv_offset=kv_offset, eps=eps, input=fused.data_ptr(), ld=fused.stride(0),
                            q_gamma=q_gamma.data_ptr(), kv_gamma=kv_gamma.data_ptr(), q_out=q_out.data_ptr(),
-                           ld_q=q_out.stride(0), tok_seq=tok_seq.data_ptr(), tok_pos=tok_pos.data_ptr(), kv=kv_view))
+                           ld_q=q_out.stride(0), tok_seq=tok_seq.data_ptr(), tok_pos=tok_pos.data_ptr(), kv=kv_view,
+                           rot_dim=rot_dim, pairing=1 if neighbours else 0, amplitude=amplitude, inv_freq=_ptr(inv_freq)))
+
+
+def latent_query(sums, heads, pitch, rot_at, rot_dim, inv_freq, tok_pos, out, neighbours=True, amplitude=1.0):
+    """out = the float32 rows ``sums`` ([tokens, heads * pitch]) in ``out``'s type, the channels
+    [rot_at, rot_at + rot_dim) of every head turned by the token's position as in ``latent_norm``."""
+    _launch(_module("latent"), "bt_latent_query_call",
+            LatentQueryCall(dtype=DTYPE_CODES[out.dtype], tokens=sums.shape[0], heads=heads, pitch=pitch, rot_at=rot_at,
+                            rot_dim=rot_dim, pairing=1 if neighbours else 0, amplitude=amplitude, input=sums.data_ptr(),
+                            ld_in=sums.stride(0), out=out.data_ptr(), ld_out=out.stride(0), inv_freq=_ptr(inv_freq),
+                            tok_pos=tok_pos.data_ptr()))
 
 
 def head_project(ctx, weight, heads, vdim, rank, head_pitch, out, gate=None):
@@ -1124,11 +1147,11 @@ def head_project(ctx, weight, heads, vdim, rank, head_pitch, out, gate=None):
 
 # --- recurrent mixers ------------------------------------------------------------------------
 
-def causal_conv(rows, weight, bias, out, state, step, cast=None):
+def causal_conv(rows, weight, bias, out, state, step, cast=None, act="silu"):
     """out = silu(bias + sum_j weight[:, j] * rows[t - (taps - 1 - j)]) per channel and sequence
-    (float32); inputs before a step's first token come from ``state`` ([slots, >= (taps - 1) *
-    channels] float32, oldest first), which then takes the step's last taps - 1 inputs.  ``cast``:
-    the same result in the products' type (zeros behind the channels)."""
+    (float32; ``act`` "none": the sum itself); inputs before a step's first token come from ``state``
+    ([slots, >= (taps - 1) * channels] float32, oldest first), which then takes the step's last taps - 1
+    inputs.  ``cast``: the same result in the products' type (zeros behind the channels)."""
     channels, taps = weight.shape
     _launch(_module("state_space"), "bt_causal_conv_call",
             CausalConvCall(cast_dtype=DTYPE_CODES[cast.dtype] if cast is not None else FLOAT32, tokens=rows.shape[0],
@@ -1137,7 +1160,8 @@ def causal_conv(rows, weight, bias, out, state, step, cast=None):
                            ld_in=rows.stride(0), weight=weight.data_ptr(), bias=_ptr(bias), out=out.data_ptr(),
                            ld_out=out.stride(0), cast=_ptr(cast), ld_cast=cast.stride(0) if cast is not None else 0,
                            state=state.data_ptr(), state_stride=state.stride(0), tok_seq=step.tok_seq.data_ptr(),
-                           seq_off=step.seq_off.data_ptr(), slots=step.slots.data_ptr()))
+                           seq_off=step.seq_off.data_ptr(), slots=step.slots.data_ptr(),
+                           act={"silu": 0, "none": 1}[act]))
 
 
 LOW_RANK_ACTS = {"softplus": 0, "sigmoid": 1, "none": 2}
@@ -1208,7 +1232,7 @@ def gated_norm(y, z, weight, parts, eps, out):
 # --- rotary positions -------------------------------------------------------------------------
 
 def head_rotary(fused, heads, kv_heads, dim, vdim, rot_dims, inv_freq, q_gamma, k_gamma, eps, q_out, tok_seq, tok_pos,
-                kv_view, dtype, neighbours=False, whole_norm=False):
+                kv_view, dtype, neighbours=False, whole_norm=False, amplitude=1.0):
     """Behind a fused query/key/value projection with float32 rows ``fused`` (queries heads * dim, keys
     kv_heads * dim, values kv_heads * vdim): every query and key head divided by its root mean square
     times ``q_gamma`` / ``k_gamma`` ([dim] float32; None: no norm), the first ``rot_dims`` channels of each
@@ -1216,14 +1240,15 @@ def head_rotary(fused, heads, kv_heads, dim, vdim, rot_dims, inv_freq, q_gamma, 
     queries go to ``q_out`` (head j at columns j * head size of the cache, zeros behind its own
     channels), keys and values into the paged cache at each token's position.
     ``neighbours``: channel 2 i turns with channel 2 i + 1 instead.  ``whole_norm``: the root mean square is
-    taken over the token's whole query (key) projection and the scales are [heads * dim] ([kv_heads * dim])."""
+    taken over the token's whole query (key) projection and the scales are [heads * dim] ([kv_heads * dim]).
+    ``amplitude``: a factor on every sine and cosine."""
     _launch(_module("rotary"), "bt_head_rotary_call",
             HeadRotaryCall(dtype=DTYPE_CODES[dtype], tokens=fused.shape[0], heads=heads, kv_heads=kv_heads, dim=dim,
                            vdim=vdim, rot_dims=rot_dims, eps=eps, input=fused.data_ptr(), ld=fused.stride(0),
                            q_gamma=_ptr(q_gamma), k_gamma=_ptr(k_gamma), inv_freq=_ptr(inv_freq),
                            q_out=q_out.data_ptr(), ld_q=q_out.stride(0), tok_seq=tok_seq.data_ptr(),
                            tok_pos=tok_pos.data_ptr(), kv=kv_view, pairing=1 if neighbours else 0,
-                           norm_span=1 if whole_norm else 0))
+                           norm_span=1 if whole_norm else 0, amplitude=amplitude))
 
 
 # --- routed feed-forward ----------------------------------------------------------------------
@@ -1243,18 +1268,24 @@ def route(h, router, correction, top, groups, keep, weights, gate_weight=None, g
                       score={"softmax": 0, "sigmoid": 1}[score], group_rank=group_rank, normalize=1 if normalize else 0))
 
 
+EXPERT_UNITS = {"gated_silu": 0, "gated_clamped": 1, "gelu_erf": 2, "silu": 3}
+
+
 def gated_experts(gu, weights, gate, experts, ff, shared_ff, identity, hidden, h=None, identity_out=None, limit=None,
-                  alpha=1.0):
+                  alpha=1.0, unit=None):
     """hidden[t, e * ff + i] = weights[t, e] * silu(gate_e,i) * up_e,i from the rows ``gu`` of a fused
     gate/up projection (per expert its gate rows, then its up rows; behind the experts the one every
     token uses, weighted by ``gate[t]``); columns behind them are set to zero.  ``identity_out`` (float32
     [rows, width]) receives (the sum of the identity experts' weights) * h.  With ``limit`` the unit is
-    g' * sigmoid(alpha * g') * (u' + 1), g' = min(gate, limit), u' = clamp(up, -limit, limit), instead of silu(gate) * up."""
+    g' * sigmoid(alpha * g') * (u' + 1), g' = min(gate, limit), u' = clamp(up, -limit, limit), instead of silu(gate) * up.
+    ``unit`` "gelu_erf" or "silu": units without a gate, act(up_e,i); ``gu`` then holds only the up rows (ff per
+    expert, the shared expert's behind them)."""
+    act = EXPERT_UNITS[unit] if unit is not None else (0 if limit is None else 1)
     _launch(_module("experts"), "bt_gated_experts_call",
             GatedExpertsCall(dtype=DTYPE_CODES[gu.dtype], tokens=gu.shape[0], experts=experts, ff=ff, shared_ff=shared_ff,
                              identity=identity, hidden_cols=hidden.shape[1], width=h.shape[1] if h is not None else 0,
                              gu=gu.data_ptr(), ld_gu=gu.stride(0), weights=_ptr(weights), gate=_ptr(gate),
-                             act=0 if limit is None else 1, limit=limit or 0.0, alpha=alpha,
+                             act=act, limit=limit or 0.0, alpha=alpha,
                              hidden=hidden.data_ptr(), ld_hidden=hidden.stride(0), h=_ptr(h),
                              ldh=h.stride(0) if h is not None else 0, identity_out=_ptr(identity_out)))
 
@@ -1303,14 +1334,16 @@ def soft_cap(logits, cap):
 # --- linear attention with a matrix state -------------------------------------------------------
 
 def keyed_scan(q, k, v, g, out, state, step, heads, kv_heads, dim, vdim, form, beta=None, A_log=None, g_bias=None,
-               lower=None, unit=False, unit_eps=1e-6, q_scale=1.0, carry=None):
+               lower=None, unit=False, unit_eps=1e-6, q_scale=1.0, carry=None, decay_per_head=False, dt_bias=None):
     """Per head S <- diag(decay) S; S <- S + key u^T; out = S^T query, token after token (csrc/linear_attention.hip).
     ``form`` "delta": u = sigmoid(beta) (v - S^T key), decay = exp(-exp(A_log) g) from step sizes ``g``, ``q`` and
     ``k`` rows of ``kv_heads`` heads (made unit vectors per head with ``unit``, q times ``q_scale``).  ``form``
     "forget": f = lower + (1 - lower) sigmoid(g + g_bias), decay = f, key = 1 - f, query = silu(q), u = v.
     ``state`` [slots, >= heads * dim * vdim rounded up to 4] float32 is read and left updated.  ``carry``: room from
     ``scan_carry`` (a slot's state floats, heads * dim extra); with it the "forget" form scans long sequences in
-    spans side by side."""
+    spans side by side.  ``decay_per_head`` ("delta"): ``g`` has one step size per head, for all its key channels;
+    ``dt_bias`` ("delta"; [heads * dim], or [heads] per head): ``g`` holds raw sums and the step size is
+    softplus(g + dt_bias)."""
     _launch(_module("linear_attention"), "bt_keyed_scan_call",
             KeyedScanCall(tokens=v.shape[0], n_seqs=step.n_seqs, heads=heads, kv_heads=kv_heads, dim=dim, vdim=vdim,
                           form={"delta": 0, "forget": 1}[form], unit=1 if unit else 0, unit_eps=unit_eps, q_scale=q_scale,
@@ -1319,14 +1352,16 @@ def keyed_scan(q, k, v, g, out, state, step, heads, kv_heads, dim, vdim, form, b
                           ld_beta=beta.stride(0) if beta is not None else 0, A_log=_ptr(A_log), g_bias=_ptr(g_bias),
                           lower=_ptr(lower), out=out.data_ptr(), ld_out=out.stride(0), S=state.data_ptr(),
                           state_stride=state.stride(0), seq_off=step.seq_off.data_ptr(), slots=step.slots.data_ptr(),
-                          span=SCAN_SPAN if carry is not None else 0, max_count=step.max_count, carry=_ptr(carry)))
+                          span=SCAN_SPAN if carry is not None else 0, max_count=step.max_count, carry=_ptr(carry),
+                          decay_span=1 if decay_per_head else 0, dt_bias=_ptr(dt_bias)))
 
 
-def head_norm_gate(y, weight, heads, vdim, eps, out, gate=None, mult=1.0):
+def head_norm_gate(y, weight, heads, vdim, eps, out, gate=None, mult=1.0, gate_act="sigmoid"):
     """out[t, h * vdim + i] = mult * y / sqrt(mean_i(y^2) + eps) * weight[i] * sigmoid(gate) per head (no last factor
-    without ``gate``, float32 logits [tokens, heads * vdim]); zeros behind the heads."""
+    without ``gate``, float32 logits [tokens, heads * vdim]; ``gate_act`` "silu": times gate * sigmoid(gate)); zeros
+    behind the heads."""
     _launch(_module("linear_attention"), "bt_head_norm_gate_call",
             HeadNormGateCall(out_dtype=DTYPE_CODES[out.dtype], tokens=y.shape[0], heads=heads, vdim=vdim,
                              out_cols=out.shape[1], eps=eps, mult=mult, y=y.data_ptr(), ld_y=y.stride(0), gate=_ptr(gate),
                              ld_gate=gate.stride(0) if gate is not None else 0, weight=weight.data_ptr(),
-                             out=out.data_ptr(), ld_out=out.stride(0)))
+                             out=out.data_ptr(), ld_out=out.stride(0), gate_act={"sigmoid": 0, "silu": 1}[gate_act]))

@@ -1,6 +1,6 @@
 """Arrangements of parts in a layer.
 
-pre_norm: y = x + mixer(norm(x)); z = y + feed_forward(norm(y))
+pre_norm: y = x + mixer(norm(x)); z = y + feed_forward(norm(y)), the feed-forward optional
 (src/models/gpt2/model.rs:218-270).  A part adds its contribution to the stream itself or
 returns it as a Delta, which stays pending until the next norm reads the stream.
 
@@ -30,12 +30,25 @@ MIXER_FOLD_ROWS = 4
 @register("block", "pre_norm")
 class PreNormBlock(Block):
     ROLES = {"mixer_norm": "norm", "mixer": "mixer", "ff_norm": "norm", "ff": "feed_forward"}
+    OPTIONAL = ("ff_norm", "ff")
     only_launches_kernels = True
+
+    def __init__(self, parts, params=None):
+        super().__init__(parts, params)
+        if ("ff" in parts) != ("ff_norm" in parts):
+            raise ValueError("pre_norm block: a feed-forward and its norm come together")
 
     def forward(self, stream, step, memory):
         parts = self.parts
-        mixer, ff, mixer_norm, ff_norm = parts["mixer"], parts["ff"], parts["mixer_norm"], parts["ff_norm"]
+        mixer, mixer_norm = parts["mixer"], parts["mixer_norm"]
         rows = stream.x.shape[0]
+        if "ff" not in parts:             # a layer that is its mixer alone
+            h = _apply(mixer_norm, stream, step, mixer.takes_deferred_norm)
+            delta = mixer.forward(h, step, memory, stream)
+            if delta is not None:
+                stream.add(delta)
+            return
+        ff, ff_norm = parts["ff"], parts["ff_norm"]
         # In a small decode step a norm can be folded into the product that follows it (one kernel
         # fewer) if the part before it leaves its output in the stream itself instead of pending
         # partial sums.  For the second norm that costs the attention output its split of K, which is

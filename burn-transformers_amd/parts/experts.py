@@ -9,10 +9,13 @@ all can), shared_ff (inner width of the expert every token uses; 0: none), score
 or "sigmoid": each router logit's own sigmoid), group_rank (a group's score is the sum of its so many best
 scores; default 1, its best), normalize (default true; false: the weights are the chosen experts' scores as
 they are), limit and alpha (with a limit an expert's unit is g' * sigmoid(alpha g') * (u' + 1) with
-g' = min(gate h, limit), u' = clamp(up h, -limit, limit), instead of silu(gate h) * (up h)).
+g' = min(gate h, limit), u' = clamp(up h, -limit, limit), instead of silu(gate h) * (up h)), unit ("gated", the
+default; "gelu_erf" or "silu": experts WITHOUT a gate, down(act(up h)), act the exact (erf) GELU or the SiLU; such
+experts have no ``gate_<e>`` / ``shared_gate`` tensors).
 Tensors: router [experts + identity, width] and correction [experts + identity] in float32, per
 expert gate / up [ff, width] and down [width, ff] (``gate_<e>``, ``up_<e>``, ``down_<e>``), and for the
-shared expert shared_gate / shared_up / shared_down and shared_mix [1, width].
+shared expert shared_gate / shared_up / shared_down and, optionally, shared_mix [1, width] (without it the shared
+expert's output is added as it is).
 
     z = router . h (32-bit), s = softmax(z) over all router outputs
     chosen = the ``top`` largest of s + correction among the open groups (a group's score is its
@@ -55,6 +58,12 @@ class RoutedExperts(FeedForward):
         self.normalize = bool(p.get("normalize", True))
         self.limit = float(p["limit"]) if p.get("limit") is not None else None
         self.alpha = float(p.get("alpha", 1.0))
+        self.unit = p.get("unit", "gated")
+        if self.unit not in ("gated", "gelu_erf", "silu"):
+            raise ValueError(f"routed experts: unknown unit {self.unit!r}")
+        if self.unit != "gated" and self.limit is not None:
+            raise ValueError("routed experts: the clamped unit has a gate")
+        self.gated = self.unit == "gated"
         if self.score not in ("softmax", "sigmoid"):
             raise ValueError(f"routed experts: unknown score {self.score!r}")
         if self.limit is not None and not self.limit > 0.0:
@@ -72,30 +81,33 @@ class RoutedExperts(FeedForward):
                              f"{(self.outputs, self.width)} in float32")
         rows, columns = [], []
         for e in range(self.experts):
-            gate, up, down = tensors[f"gate_{e}"], tensors[f"up_{e}"], tensors[f"down_{e}"]
+            up, down = tensors[f"up_{e}"], tensors[f"down_{e}"]
+            gate = tensors[f"gate_{e}"] if self.gated else up
             if tuple(gate.shape) != (self.ff, self.width) or tuple(up.shape) != (self.ff, self.width) or \
                     tuple(down.shape) != (self.width, self.ff):
                 raise ValueError(f"routed experts: expert {e}'s matrices do not have the configured sizes")
-            rows += [gate, up]
+            rows += [gate, up] if self.gated else [up]
             columns.append(down)
         self.shared_mix = None
         if self.shared_ff:
-            gate, up, down = tensors["shared_gate"], tensors["shared_up"], tensors["shared_down"]
+            up, down = tensors["shared_up"], tensors["shared_down"]
+            gate = tensors["shared_gate"] if self.gated else up
             if tuple(gate.shape) != (self.shared_ff, self.width) or tuple(up.shape) != (self.shared_ff, self.width) or \
                     tuple(down.shape) != (self.width, self.shared_ff):
                 raise ValueError("routed experts: the shared expert's matrices do not have the configured sizes")
-            rows += [gate, up]
+            rows += [gate, up] if self.gated else [up]
             columns.append(down)
-            self.shared_mix = tensors["shared_mix"].reshape(-1).contiguous()
-            if tuple(self.shared_mix.shape) != (self.width,) or self.shared_mix.dtype != torch.float32:
-                raise ValueError("routed experts: the shared expert's gate is one float32 row of the model's width")
+            if "shared_mix" in tensors:
+                self.shared_mix = tensors["shared_mix"].reshape(-1).contiguous()
+                if tuple(self.shared_mix.shape) != (self.width,) or self.shared_mix.dtype != torch.float32:
+                    raise ValueError("routed experts: the shared expert's gate is one float32 row of the model's width")
         if not rows:
             raise ValueError("routed experts: no expert has tensors")
         dtype = rows[0].dtype
         self.inner = self.experts * self.ff + self.shared_ff
         self.hidden_cols = operand_columns(self.inner, dtype)
-        self.fused_cols = operand_columns(2 * self.inner, dtype)      # (rows of the fused product's output start where 16-byte stores may)
-        # [2 * inner (+ zero rows), width (+ zero columns, where the rows it multiplies carry them)]
+        self.fused_cols = operand_columns((2 if self.gated else 1) * self.inner, dtype)      # (rows of the fused product's output start where 16-byte stores may)
+        # [2 * inner, or inner without gates (+ zero rows), width (+ zero columns, where the rows it multiplies carry them)]
         self.in_weight = pad_columns(pad_rows(torch.cat(rows), self.fused_cols), operand_columns(self.width, dtype))
         self.down_weight = pad_columns(torch.cat(columns, dim=1), self.hidden_cols)           # [width, inner (+ zeros)]
         on_gpu = self.in_weight.is_cuda
@@ -108,7 +120,7 @@ class RoutedExperts(FeedForward):
     def forward(self, h, step, stream):
         tokens = h.shape[0]
         weights = step.buffer("experts.weights", tokens, self.outputs, "float32")
-        mix = step.buffer("experts.mix", tokens, 1, "float32") if self.shared_ff else None
+        mix = step.buffer("experts.mix", tokens, 1, "float32") if self.shared_mix is not None else None
         K.route(h, self.router, self.correction, self.top, self.groups, self.keep, weights, self.shared_mix, mix,
                 score=self.score, group_rank=self.group_rank, normalize=self.normalize)
         fused = step.buffer("experts.fused", tokens, self.fused_cols, step.dtype)
@@ -119,6 +131,6 @@ class RoutedExperts(FeedForward):
         partials = step.partial_sums("experts.partials", splits + extra, tokens, self.width)
         K.gated_experts(fused, weights, mix, self.experts, self.ff, self.shared_ff, self.identity, hidden,
                         h=h if self.identity else None, identity_out=partials[splits] if self.identity else None,
-                        limit=self.limit, alpha=self.alpha)
+                        limit=self.limit, alpha=self.alpha, unit=None if self.gated else self.unit)
         K.gemm(hidden, self.down_weight, K.epilogue_f32(partials[:splits]), splits=splits, packed=self.down_packed)
         return Delta(partials, None)

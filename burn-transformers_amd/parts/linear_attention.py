@@ -12,6 +12,10 @@ a2 [heads * dim, r], dt_bias [heads * dim], A_log [heads], g1 [r', width], g2 [h
     beta = sigmoid(beta_weight h);   g = exp(-exp(A_log) * softplus(a2 (a1 h) + dt_bias))  per head and key channel
     S <- diag(g) S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q
     out = out_weight (o / rms(o over vdim) * norm_weight * sigmoid(g2 (g1 h)))
+  Parameters of the rule's variants: low_rank (default true; false: the step sizes' and the output gate's projections
+  are single matrices ``a_weight`` and ``g_weight`` in place of a1, a2 and g1, g2), decay_span ("channel", the
+  default, or "head": ONE decay per head for all its key channels, a_weight [heads, width], dt_bias [heads]),
+  gate_act ("sigmoid", the default, or "silu": the output is multiplied by z sigmoid(z) of the gate's sums z).
 
 forget_gate_attention: parameters width, heads, dim, vdim, eps.  Tensors: q_weight, f_weight [heads * dim,
 width], f_bias, lower [heads * dim], v_weight [heads * vdim, width], norm_weight [vdim], out_weight.
@@ -93,23 +97,35 @@ class GatedDeltaRule(_MatrixState):
         self._sizes(params)
         self.kv_heads, self.taps = params["kv_heads"], int(params["taps"])
         self.unit_eps = float(params.get("unit_eps", 1e-6))
+        self.low_rank = bool(params.get("low_rank", True))
+        self.per_head = {"channel": False, "head": True}[params.get("decay_span", "channel")]
+        self.gate_act = params.get("gate_act", "sigmoid")
+        if self.gate_act not in ("sigmoid", "silu"):
+            raise ValueError(f"gated_delta_rule: unknown activation {self.gate_act!r} of the output gate")
         if self.heads % self.kv_heads != 0:
             raise ValueError(f"gated_delta_rule: {self.heads} heads cannot share {self.kv_heads} heads of queries and keys")
         qk, t = self.kv_heads * self.dim, tensors
-        self.rank_a, self.rank_g = t["a1"].shape[0], t["g1"].shape[0]
-        _check("gated_delta_rule", t, {
-            "q_weight": (qk, self.width), "k_weight": (qk, self.width), "v_weight": (self.inner, self.width),
-            "q_conv": (qk, self.taps), "k_conv": (qk, self.taps), "v_conv": (self.inner, self.taps),
-            "beta_weight": (self.heads, self.width), "a1": (self.rank_a, self.width),
-            "a2": (self.heads * self.dim, self.rank_a), "dt_bias": (self.heads * self.dim,), "A_log": (self.heads,),
-            "g1": (self.rank_g, self.width), "g2": (self.inner, self.rank_g), "norm_weight": (self.vdim,),
-            "out_weight": (self.width, self.inner)})
+        self.decays = self.heads if self.per_head else self.heads * self.dim
+        shapes = {"q_weight": (qk, self.width), "k_weight": (qk, self.width), "v_weight": (self.inner, self.width),
+                  "q_conv": (qk, self.taps), "k_conv": (qk, self.taps), "v_conv": (self.inner, self.taps),
+                  "beta_weight": (self.heads, self.width), "dt_bias": (self.decays,), "A_log": (self.heads,),
+                  "norm_weight": (self.vdim,), "out_weight": (self.width, self.inner)}
+        if self.low_rank:
+            self.rank_a, self.rank_g = t["a1"].shape[0], t["g1"].shape[0]
+            shapes.update(a1=(self.rank_a, self.width), a2=(self.decays, self.rank_a), g1=(self.rank_g, self.width),
+                          g2=(self.inner, self.rank_g))
+        else:
+            self.rank_a, self.rank_g = self.decays, self.inner          # the fused product's columns are the sums themselves
+            shapes.update(a_weight=(self.decays, self.width), g_weight=(self.inner, self.width))
+        _check("gated_delta_rule", t, shapes)
         self.qk, self.channels = qk, 2 * qk + self.inner
         self.at_beta = self.channels
         self.at_a, self.at_g = self.at_beta + self.heads, self.at_beta + self.heads + self.rank_a
-        self._finish([t["q_weight"], t["k_weight"], t["v_weight"], t["beta_weight"], t["a1"], t["g1"]], t["out_weight"])
+        first, second = (t["a1"], t["g1"]) if self.low_rank else (t["a_weight"], t["g_weight"])
+        self._finish([t["q_weight"], t["k_weight"], t["v_weight"], t["beta_weight"], first, second], t["out_weight"])
         self.conv_weight = torch.cat([t["q_conv"], t["k_conv"], t["v_conv"]]).float().contiguous()
-        self.a2, self.g2 = t["a2"].contiguous(), t["g2"].contiguous()
+        if self.low_rank:
+            self.a2, self.g2 = t["a2"].contiguous(), t["g2"].contiguous()
         self.dt_bias, self.A_log, self.norm_weight = t["dt_bias"], t["A_log"], t["norm_weight"]
         self.conv_state = (self.taps - 1) * self.channels
 
@@ -120,16 +136,20 @@ class GatedDeltaRule(_MatrixState):
         fused = self._project(h, step, "delta.in")
         qkv = step.buffer("delta.qkv", tokens, self.channels, "float32")
         K.causal_conv(fused[:, :self.channels], self.conv_weight, None, qkv, conv_state, step)
-        dt = step.buffer("delta.dt", tokens, self.heads * self.dim, "float32")
-        K.dt_project(fused[:, self.at_a:self.at_a + self.rank_a], self.a2, self.dt_bias, dt, act="softplus")
-        gate = step.buffer("delta.gate", tokens, self.inner, "float32")
-        K.dt_project(fused[:, self.at_g:self.at_g + self.rank_g], self.g2, None, gate, act="none")
+        if self.low_rank:
+            dt = step.buffer("delta.dt", tokens, self.decays, "float32")
+            K.dt_project(fused[:, self.at_a:self.at_a + self.rank_a], self.a2, self.dt_bias, dt, act="softplus")
+            gate = step.buffer("delta.gate", tokens, self.inner, "float32")
+            K.dt_project(fused[:, self.at_g:self.at_g + self.rank_g], self.g2, None, gate, act="none")
+            raw = None
+        else:            # the sums are in the fused product's rows: the scan adds the bias and takes the softplus itself
+            dt, gate, raw = fused[:, self.at_a:self.at_a + self.decays], fused[:, self.at_g:self.at_g + self.inner], self.dt_bias
         y = step.buffer("delta.y", tokens, self.inner, "float32")
         K.keyed_scan(qkv[:, :qk], qkv[:, qk:2 * qk], qkv[:, 2 * qk:], dt, y, scan_state, step, self.heads, self.kv_heads,
                      self.dim, self.vdim, "delta", beta=fused[:, self.at_beta:self.at_beta + self.heads], A_log=self.A_log,
-                     unit=True, unit_eps=self.unit_eps, q_scale=self.dim ** -0.5)
+                     unit=True, unit_eps=self.unit_eps, q_scale=self.dim ** -0.5, decay_per_head=self.per_head, dt_bias=raw)
         gated = step.buffer("delta.gated", tokens, self.inner_cols, step.dtype)
-        K.head_norm_gate(y, self.norm_weight, self.heads, self.vdim, self.eps, gated, gate=gate)
+        K.head_norm_gate(y, self.norm_weight, self.heads, self.vdim, self.eps, gated, gate=gate, gate_act=self.gate_act)
         stream.add_product(step, gated, self.out_weight, packed=self.out_packed)
 
 
