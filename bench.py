@@ -1,7 +1,7 @@
 """Throughput of GPT-2 generation on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers 48] [--dtype bf16]
-                    [--repetitions 10] [--workload xl|small|medium|sweep|salopel|kodatar|rotutar] [--model xl|medium|small]
+                    [--repetitions 10] [--workload xl|small|medium|sweep|salopel|kodatar|rotutar|gavasun] [--model xl|medium|small]
                     [--kernel-batches 1,64] [--sweep-part all|decode|prompts] [--no-points] [--no-kernels] [--no-own]
 
 The default workload (``xl``) has the layer sizes of GPT-2 XL with random weights: a batch of 8
@@ -52,6 +52,9 @@ experts, a stretch of layers that runs twice), beside GPT-2 at equal width, runs
 ``--workload rotutar`` runs the fourth family, Rotutar (linear attention with a matrix state, window attention
 with a sink beside a delta rule, gated sublayer outputs, routed experts), beside Salopel, the library's closest
 family, at equal width, layers and vocabulary.
+``--workload gavasun`` runs the fifth family, Gavasun (chunk attention behind short convolutions, latent attention
+with a shared turned key part in a window, a delta rule with one decay a head, ungated experts), beside Rotutar,
+the library's closest family, at equal width, layers and vocabulary.
 """
 
 import argparse
@@ -206,7 +209,9 @@ def _class_of(name, call):
     if short == "poly_norm":
         return f"poly_norm {call.tokens}x{call.columns}", call.tokens * call.columns * 6, 0.0
     if short == "latent_norm":
-        return f"latent_norm {call.tokens}tok", call.tokens * (call.q_rank + call.kv_rank) * 8, 0.0
+        return f"latent_norm {call.tokens}tok", call.tokens * (call.q_rank + call.kv_rank + call.rot_dim) * 8, 0.0
+    if short == "latent_query":
+        return f"latent_query {call.tokens}x{call.heads * call.pitch}", call.tokens * call.heads * call.pitch * (4 + (4 if call.dtype == 0 else 2)), 0.0
     if short == "head_project":
         element = 4 if call.dtype == 0 else 2
         work = call.heads * call.vdim * call.rank
@@ -608,6 +613,36 @@ def rotutar_config(width, layers, vocab):
             "layers": [dict(group[i % 4]) for i in range(layers)]}
 
 
+def gavasun_config(width, layers, vocab):
+    """Gavasun at layer sizes that resemble a real model's: groups of four layers (chunk attention with a dense
+    feed-forward of 4 x width, a delta rule with experts, latent attention with experts, a delta rule with experts);
+    heads of 128 everywhere, the attention's on a quarter as many key/value heads, half of every head turned, chunks of
+    512, four taps; the delta rule's queries and keys on half as many heads, four taps; the latent attention's heads
+    of 128 plain and 32 turned channels on a key/value latent of 96 (a cached head of 128) and a query latent of 3/8 of
+    the width, a window of 512; eight experts of the model's width of which a token uses two, and one every token uses."""
+    heads = max(4, width // 128)
+    slowed = {"factor": 8.0, "original": 2048, "fast": 32.0, "slow": 1.0}
+    attention = {"heads": heads, "kv_heads": heads // 4, "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "conv": 4,
+                 "rot": {"dims": 64, "base": 1000000.0, "scaling": slowed}, "mask": {"size": 512}}
+    delta = {"heads": heads, "kv_heads": heads // 2, "dim": 128, "vdim": 128, "conv": 4}
+    latent = {"heads": min(heads, 16), "dim": 128, "rot_dim": 32, "vdim": 128, "q_rank": 3 * width // 8, "kv_rank": 96,
+              "scale": 160 ** -0.5, "rot": {"dims": 32, "base": 20000.0, "scaling": slowed}, "mask": {"size": 512}}
+    experts = {"kind": "moe", "expert": {"ff": width}, "router": {"experts": 8, "top": 2}, "shared": {"ff": width}}
+    group = [{"type": "attention", "mixer": attention, "mlp": {"kind": "dense", "ff": 4 * width}},
+             {"type": "delta", "mixer": delta, "mlp": experts}, {"type": "latent_attention", "mixer": latent, "mlp": experts},
+             {"type": "delta", "mixer": delta, "mlp": experts}]
+    return {"architecture": "Gavasun", "vocab": vocab, "width": width, "embedding": {"scale": 1.0}, "norm": {"eps": 1e-5},
+            "loop": None, "layers": [dict(group[i % 4]) for i in range(layers)]}
+
+
+def run_gavasun(args):
+    """Gavasun beside the library's closest family, Rotutar (a delta rule with a matrix state, rotary attention on
+    grouped heads, routed experts), at equal width, layers and vocabulary."""
+    heads = lambda width: max(4, width // 128)
+    sizes = lambda width: (2 * 128 * (heads(width) // 4), 128 * heads(width))
+    run_beside_gpt2(args, "gavasun", gavasun_config, sizes, other=("rotutar", rotutar_config, sizes))
+
+
 def run_rotutar(args):
     """Rotutar beside the library's closest family, Salopel (recurrent layers with a state per sequence, norms of
     the sublayers' outputs), at equal width, layers and vocabulary."""
@@ -698,7 +733,7 @@ def main():
     parser.add_argument("--kernel-batches", default="", help="further batch sizes whose decode kernel classes are timed, e.g. 1,64")
     parser.add_argument("--dtype", choices=["bf16", "fp32"], default=None)
     parser.add_argument("--repetitions", type=int, default=10, help="measured repetitions, each on fresh sequences")
-    parser.add_argument("--workload", choices=["xl", "small", "medium", "sweep", "salopel", "kodatar", "rotutar"], default="xl")
+    parser.add_argument("--workload", choices=["xl", "small", "medium", "sweep", "salopel", "kodatar", "rotutar", "gavasun"], default="xl")
     parser.add_argument("--sweep-part", choices=["all", "decode", "prompts"], default="all",
                         help="which table of --workload sweep to run")
     parser.add_argument("--no-points", action="store_true", help="skip batch 1 and 64")
@@ -711,8 +746,8 @@ def main():
     if args.repetitions < 1:
         parser.error("--repetitions must be at least 1")
     args.kernel_batches = [int(b) for b in args.kernel_batches.split(",") if b]
-    if args.workload in ("salopel", "kodatar", "rotutar"):
-        {"salopel": run_salopel, "kodatar": run_kodatar, "rotutar": run_rotutar}[args.workload](args)
+    if args.workload in ("salopel", "kodatar", "rotutar", "gavasun"):
+        {"salopel": run_salopel, "kodatar": run_kodatar, "rotutar": run_rotutar, "gavasun": run_gavasun}[args.workload](args)
         return
     if args.layers is None:
         args.layers = XL["n_layer"] if args.workload == "sweep" else MODELS[args.model]["n_layer"]

@@ -79,7 +79,9 @@ class LatentAttention(Mixer):
         self.fused_cols = self.gate_offset + (self.heads * self.vdim if self.gated else 0)
         self.fused_weight = torch.cat([pad_rows(tensors["down_q"], self.kv_offset),
                                        pad_rows(tensors["down_kv"], self.gate_offset - self.kv_offset)] +
-                                      ([tensors["gate"]] if self.gated else [])).contiguous()
+                                      ([tensors["gate"]] if self.gated else []))
+        # (the rows it multiplies carry zero columns where the width is no multiple of what 16-byte loads take)
+        self.fused_weight = pad_columns(self.fused_weight, operand_columns(self.width, dtype))
         self.q_norm, self.kv_norm = tensors["q_norm"], tensors["kv_norm"]
         # absorbed queries: rows i * head_dim .. of W are up_k_i^T up_q_i  ([kv_rank, q_rank]), and behind them
         # the head's turned rows of up_q as they are

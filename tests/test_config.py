@@ -64,7 +64,7 @@ def test_registry_resolves_architectures_first_then_model_type():
     family = bt.resolve_family({"architectures": ["GPT2LMHeadModel"]})
     assert family.name == "gpt2" and family is bt.resolve_family({"model_type": "gpt2"})
     assert family is bt.resolve_family({"architectures": ["SomethingElse"], "model_type": "gpt2"})
-    with pytest.raises(bt.UnsupportedArchitecture, match="`LlamaForCausalLM`.*supported values: GPT2LMHeadModel, Kodatar, Rotutar, Salopel, gpt2, kodatar, rotutar, salopel"):
+    with pytest.raises(bt.UnsupportedArchitecture, match="`LlamaForCausalLM`.*supported values: GPT2LMHeadModel, Gavasun, Kodatar, Rotutar, Salopel, gavasun, gpt2, kodatar, rotutar, salopel"):
         bt.resolve_family({"architectures": ["LlamaForCausalLM"], "model_type": "llama"})
     with pytest.raises(bt.UnsupportedArchitecture, match="nothing"):
         bt.resolve_family({})
