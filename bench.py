@@ -196,7 +196,8 @@ def _class_of(name, call):
         rows = call.M * call.K * (4 if call.has_norm else element)
         return f"{short} {call.M}x{call.N}x{call.K}", weights + rows, 2.0 * call.M * call.N * call.K
     if short.startswith("attention"):
-        return f"{short} {call.args.n_tokens}tok", None, None       # filled in by the caller, who knows the contexts
+        args = call.args                                           # (bytes and flops are filled in by the caller, who knows the contexts)
+        return f"{short} {args.n_tokens}tok {args.q_heads}x{args.kv.head_dim} on {args.kv.kv_heads}", None, None
     if short == "add_norm":
         return f"add_norm {call.n_rows}x{call.width}", (call.n_delta + 2) * call.n_rows * call.width * 4, 0.0
     if short == "embed":

@@ -119,6 +119,9 @@ __global__ void __launch_bounds__(KS_THREADS) keyed_scan_kernel(KeyedScanCall c,
   float* Kp = lds + (size_t)2 * chunk * NP;                                   // [chunk][NP] keys (delta rule)
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, sub = lane & 15, pl = lane >> 4;
   float2* tok = reinterpret_cast<float2*>(lds + (size_t)PLANES * chunk * NP) + (size_t)wave * chunk * 4;   // [waves][chunk][4]: v, beta
+  // one decay a head: a run's decays are worked out once a token (thread i takes token i), not once a key channel
+  float* dec = lds + (size_t)PLANES * chunk * NP + (size_t)KS_WAVES * chunk * 8;                          // [chunk]
+  const bool per_head = FORM == 0 && c.decay_span == 1;
   const int tile = min((int)blockIdx.x * KS_WAVES + wave, tiles - 1), head = blockIdx.y;
   const int seq = blockIdx.z % c.n_seqs, part = blockIdx.z / c.n_seqs;
   const bool works = (int)blockIdx.x * KS_WAVES + wave < tiles;
@@ -162,14 +165,14 @@ __global__ void __launch_bounds__(KS_THREADS) keyed_scan_kernel(KeyedScanCall c,
   if (raw_steps) bias = c.dt_bias[col_g];
   const int ch = tile * 4 + (lane & 3);                   // the value channel of a lane's (v, beta) pairs
   const int chc = ch < c.vdim ? ch : 0;
-  float rg[KS_LOADS], rk[KS_LOADS], rq[KS_LOADS], rv[TOK_LOADS], rb[TOK_LOADS];
+  float rg[KS_LOADS], rk[KS_LOADS], rq[KS_LOADS], rv[TOK_LOADS], rb[TOK_LOADS], rh = 0.f;
   // issues the loads of the run that starts at token t0 (rows beyond the run read its last token and are dropped)
   auto fetch = [&](int t0, int count) {
 #pragma unroll
     for (int j = 0; j < KS_LOADS; ++j) {
       const int i = min(row0 + j * ROWS_A_TURN, count - 1);
       const int64_t t = t0 + i;
-      rg[j] = c.g[t * c.ld_g + col_g];
+      rg[j] = per_head ? 0.f : c.g[t * c.ld_g + col_g];
       rq[j] = PHASE == 1 ? 0.f : c.q[t * c.ld_q + (FORM == 0 ? col_k : col_g)];
       rk[j] = FORM == 0 ? c.k[t * c.ld_k + col_k] : 0.f;
     }
@@ -180,11 +183,16 @@ __global__ void __launch_bounds__(KS_THREADS) keyed_scan_kernel(KeyedScanCall c,
       rv[j] = c.v[t * c.ld_v + head * c.vdim + chc];
       rb[j] = FORM == 0 ? c.beta[t * c.ld_beta + head] : 0.f;
     }
+    if (per_head) rh = c.g[(int64_t)(t0 + min((int)threadIdx.x, count - 1)) * c.ld_g + head];
   };
   if (first < last) fetch(first, min(chunk, last - first));
   for (int t0 = first; t0 < last; t0 += chunk) {
     const int count = min(chunk, last - t0);
     __syncthreads();                                       // the run before has been walked
+    if (per_head) {
+      if ((int)threadIdx.x < count) dec[threadIdx.x] = expf(rate * (raw_steps ? softplus_f(rh + bias) : rh));
+      __syncthreads();
+    }
 #pragma unroll
     for (int j = 0; j < KS_LOADS; ++j) {
       const int i = row0 + j * ROWS_A_TURN;
@@ -192,7 +200,7 @@ __global__ void __launch_bounds__(KS_THREADS) keyed_scan_kernel(KeyedScanCall c,
         float decay = 0.f, query = 0.f;
         if (in_head) {
           if (FORM == 0) {
-            decay = expf(rate * (raw_steps ? softplus_f(rg[j] + bias) : rg[j]));
+            decay = per_head ? dec[i] : expf(rate * (raw_steps ? softplus_f(rg[j] + bias) : rg[j]));
             query = rq[j];
           } else {
             decay = low + (1.0f - low) / (1.0f + expf(-(rg[j] + bias)));
@@ -321,7 +329,7 @@ __global__ void __launch_bounds__(256) keyed_carry_kernel(KeyedScanCall c, int t
 
 template <int R>
 static void launch_keyed_scan(hipStream_t stream, const KeyedScanCall& c) {
-  const int per_token = (c.form == 0 ? 3 : 2) * 16 * R + 8 * KS_WAVES;
+  const int per_token = (c.form == 0 ? 3 : 2) * 16 * R + 8 * KS_WAVES + 1;      // planes, (v, beta) pairs, a decay
   const int tiles = (c.vdim + 3) / 4, groups = (tiles + KS_WAVES - 1) / KS_WAVES;
   dim3 block(KS_THREADS);
   const int span = c.form == 1 ? span_tokens(c.span, c.max_count, c.carry, (int64_t)groups * KS_WAVES * c.heads * c.n_seqs, 1) : 0;
