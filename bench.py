@@ -622,12 +622,12 @@ def gavasun_config(width, layers, vocab):
     of 128 plain and 32 turned channels on a key/value latent of 96 (a cached head of 128) and a query latent of 3/8 of
     the width, a window of 512; eight experts of the model's width of which a token uses two, and one every token uses."""
     heads = max(4, width // 128)
-    slowed = {"factor": 8.0, "original": 2048, "fast": 32.0, "slow": 1.0}
+    slowed = {"factor": 4.0, "original": 2048, "fast": 16.0, "slow": 2.0}
     attention = {"heads": heads, "kv_heads": heads // 4, "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "conv": 4,
-                 "rot": {"dims": 64, "base": 1000000.0, "scaling": slowed}, "mask": {"size": 512}}
+                 "rot": {"dims": 64, "base": 500000.0, "scaling": slowed}, "mask": {"size": 512}}
     delta = {"heads": heads, "kv_heads": heads // 2, "dim": 128, "vdim": 128, "conv": 4}
     latent = {"heads": min(heads, 16), "dim": 128, "rot_dim": 32, "vdim": 128, "q_rank": 3 * width // 8, "kv_rank": 96,
-              "scale": 160 ** -0.5, "rot": {"dims": 32, "base": 20000.0, "scaling": slowed}, "mask": {"size": 512}}
+              "scale": 160 ** -0.5, "rot": {"dims": 32, "base": 10000.0, "scaling": slowed}, "mask": {"size": 512}}
     experts = {"kind": "moe", "expert": {"ff": width}, "router": {"experts": 8, "top": 2}, "shared": {"ff": width}}
     group = [{"type": "attention", "mixer": attention, "mlp": {"kind": "dense", "ff": 4 * width}},
              {"type": "delta", "mixer": delta, "mlp": experts}, {"type": "latent_attention", "mixer": latent, "mlp": experts},

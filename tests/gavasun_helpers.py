@@ -64,15 +64,15 @@ ODD = model_config([layer(delta(3, 1, 20, 12, 1), moe(5, 12, 1)),
                     layer(latent(2, 12, 0, 20, 30, 20, 0.3), dense(22)),
                     layer(delta(2, 2, 40, 8, 2))], width=40, vocab=97, eps=1e-3, scale=0.5, loop=(0, 2, 3))
 # each mechanism alone, in a model of one layer
-ATTENTION_ONLY = model_config([layer(attention(4, 2, 32, 32, 0.18, taps=4, rot=rotation(16, 1000.0, (8.0, 32, 32.0, 1.0)), chunk=40))],
+ATTENTION_ONLY = model_config([layer(attention(4, 2, 32, 32, 0.18, taps=4, rot=rotation(16, 1000.0, (6.0, 32, 24.0, 1.0)), chunk=40))],
                               vocab=101)
 LATENT_ONLY = model_config([layer(latent(4, 32, 16, 24, 48, 64, 0.15, base=5000.0, scaling=(4.0, 64, 16.0, 1.0), window=33))], vocab=101)
 DELTA_ONLY = model_config([layer(delta(4, 2, 24, 16, 4))], vocab=101)
 DENSE_ONLY = model_config([layer(delta(1, 1, 8, 8, 2), dense(72))], width=32, vocab=61)
 EXPERTS_ONLY = model_config([layer(delta(1, 1, 8, 8, 2), moe(8, 16, 2, shared=24))], width=32, vocab=61)
 # chunks and windows that span several blocks of the cache, heads of 128, a latent wider than any MFMA attention kernel's head
-LONG = model_config([layer(attention(2, 1, 128, 64, 0.09, taps=4, rot=rotation(64, 300000.0, (8.0, 256, 32.0, 1.0)), chunk=200), dense(64)),
-                     layer(latent(2, 64, 32, 48, 64, 112, 0.1, base=20000.0, scaling=(2.0, 512, 32.0, 1.0), window=150), moe(4, 32, 2, shared=16)),
+LONG = model_config([layer(attention(2, 1, 128, 64, 0.09, taps=4, rot=rotation(64, 300000.0, (5.0, 256, 24.0, 1.5)), chunk=200), dense(64)),
+                     layer(latent(2, 64, 32, 48, 64, 112, 0.1, base=30000.0, scaling=(3.0, 512, 16.0, 1.0), window=150), moe(4, 32, 2, shared=16)),
                      layer(delta(2, 2, 128, 32, 4))], width=96, vocab=151)
 # a latent whose cached head fits the MFMA kernels (96 + 32), more query heads on a cached head than a decode tile takes
 NARROW_LATENT = model_config([layer(latent(4, 32, 32, 32, 48, 96, 0.12, window=70), dense(48)),
@@ -179,7 +179,7 @@ def random_config(seed):
             dim, rot_dim = rng.choice([16, 32, 64, 96]), rng.choice([0, 8, 16, 32, 64])
             mixer = latent(rng.choice([1, 2, 4, 8]), dim, rot_dim, rng.choice([16, 32, 48, 80]), rng.choice([24, 64, 96]),
                            rng.choice([32, 64, 96, 128, 192]), (dim + rot_dim) ** -0.5 * rng.choice([0.7, 1.0, 1.5]),
-                           base=rng.choice([100.0, 20000.0]), scaling=scaling(),
+                           base=rng.choice([100.0, 30000.0]), scaling=scaling(),
                            window=rng.choice([5, 32, 64, 96, 100, 160]) if rng.random() < 0.85 else None)
         else:
             shared = rng.choice([1, 2, 4])

@@ -125,7 +125,7 @@ def test_slowed_frequencies():
     assert all(got[i] <= plain_f[i] and got[i] >= plain_f[i] / 4.0 for i in range(dims // 2))
     assert rotary_amplitude(scaling) == pytest.approx(0.1 * math.log(4.0) + 1.0) and rotary_amplitude(None) == 1.0
     assert torch.equal(rotary_frequencies(dims, base, None), plain_f)
-    for rot in ({"dims": 32, "base": 1e6, "scaling": {"factor": 8.0, "original": 512, "fast": 32.0, "slow": 1.0}},
+    for rot in ({"dims": 24, "base": 3e5, "scaling": {"factor": 5.0, "original": 300, "fast": 20.0, "slow": 1.5}},
                 {"dims": 6, "base": 50.0, "scaling": {"factor": 2.0, "original": 16, "fast": 2.0, "slow": 0.25}}):
         f, amplitude = plain.frequencies(rot)
         assert torch.allclose(rotary_frequencies(rot["dims"], rot["base"], rot["scaling"]), f, rtol=1e-13, atol=0.0)

@@ -118,11 +118,11 @@ def test_convolution_without_activation_in_portions(taps):
         assert rel_err(g, w) < 1e-6
 
 
-SCALINGS = [None, {"factor": 8.0, "original": 64, "fast": 32.0, "slow": 1.0}, {"factor": 2.0, "original": 4096, "fast": 4.0, "slow": 0.5}]
+SCALINGS = [None, {"factor": 6.0, "original": 64, "fast": 24.0, "slow": 1.0}, {"factor": 3.0, "original": 4096, "fast": 4.0, "slow": 0.5}]
 
 
 @pytest.mark.parametrize("scaling", SCALINGS)
-@pytest.mark.parametrize("dims,base", [(32, 1000000.0), (6, 50.0), (64, 20000.0)])
+@pytest.mark.parametrize("dims,base", [(32, 300000.0), (6, 50.0), (64, 7000.0)])
 def test_frequencies_and_amplitude(dims, base, scaling):
     rot = {"dims": dims, "base": base, "scaling": scaling}
     f, amplitude = plain.frequencies(rot)
